@@ -16,7 +16,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..parts.needs import PagedNeed, StateNeed
+from ..parts.needs import PagedNeed, StateNeed, each_need
 from .manager import GroupSpec
 
 
@@ -43,7 +43,14 @@ def plan_groups(cache_needs: list) -> tuple[list[GroupSpec], list[PagedNeed], li
                 needs.append(need)
             of_entry.append(needs.index(need))
         else:
-            of_entry.append(None)
+            # (an entry whose mixer is made of several: its paged needs join their groups; ``of_entry`` names the first)
+            first = None
+            for single in each_need(need) if isinstance(need, (tuple, list)) else ():
+                if isinstance(single, PagedNeed):
+                    if single not in needs:
+                        needs.append(single)
+                    first = needs.index(single) if first is None else first
+            of_entry.append(first)
     specs = [GroupSpec(n.group_name, n.window) for n in needs]
     return specs, needs, of_entry
 
@@ -52,7 +59,9 @@ class CacheStorage:
     def __init__(self, model, num_pages: list[int], page_size: int, num_slots: int, dtype, device) -> None:
         self.group_specs, needs, of_entry = plan_groups(model.cache_needs)
         self.page_size = page_size
-        counts = [sum(1 for g in of_entry if g == i) for i in range(len(needs))]
+        flat = [(single, i) for i, (need, call) in enumerate(zip(model.cache_needs, model.spec.run_order)) if call.cache_from is None
+                for single in each_need(need)]
+        counts = [sum(1 for single, _ in flat if isinstance(single, PagedNeed) and needs.index(single) == i) for i in range(len(needs))]
         self.k = [torch.zeros((counts[i], num_pages[i], n.kv_heads, page_size, n.head_dim), dtype=dtype, device=device)
                   for i, n in enumerate(needs)]
         self.v = [torch.zeros((counts[i], num_pages[i], n.kv_heads, n.v_dim, page_size), dtype=dtype, device=device)
@@ -60,19 +69,22 @@ class CacheStorage:
         self.states: list[torch.Tensor] = []
         self.views: list = []
         taken = [0] * len(needs)
-        for i, (need, call) in enumerate(zip(model.cache_needs, model.spec.run_order)):
-            if call.cache_from is not None:
-                self.views.append(self.views[call.cache_from])
-            elif isinstance(need, PagedNeed):
-                g = of_entry[i]
-                self.views.append(PagedView(g, self.k[g][taken[g]], self.v[g][taken[g]]))
+        def view_of(need):
+            if isinstance(need, (tuple, list)):
+                return tuple(view_of(single) for single in need)
+            if isinstance(need, PagedNeed):
+                g = needs.index(need)
+                view = PagedView(g, self.k[g][taken[g]], self.v[g][taken[g]])
                 taken[g] += 1
-            elif isinstance(need, StateNeed):
+                return view
+            if isinstance(need, StateNeed):
                 t = torch.zeros((num_slots, *need.shape), dtype=need.dtype, device=device)
                 self.states.append(t)
-                self.views.append(StateView(t))
-            else:
-                self.views.append(None)
+                return StateView(t)
+            return None
+
+        for i, (need, call) in enumerate(zip(model.cache_needs, model.spec.run_order)):
+            self.views.append(self.views[call.cache_from] if call.cache_from is not None else view_of(need))
         # state that belongs to the model and to no layer (``model.state_needs``: name -> StateNeed)
         self.model_state: dict[str, torch.Tensor] = {}
         for name, need in getattr(model, "state_needs", {}).items():

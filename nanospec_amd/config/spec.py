@@ -27,6 +27,15 @@ class RMSNormSpec:
 
 
 @dataclass(frozen=True)
+class NoNormSpec:
+    """No norm: y = x.  In front of a sublayer of a block over a 32-bit stream it means that the sublayer reads the stream
+    itself (rounded to the model's precision)."""
+
+    kind: ClassVar[str] = "none"
+    dim: int
+
+
+@dataclass(frozen=True)
 class RopeSpec:
     """Rotary position encoding over the first ``rotary_dim`` elements of a head; pair j is elements j and
     j + rotary_dim/2 (``interleaved``: 2j and 2j + 1).  ``scaling`` is None or the llama3 frequency scaling as
@@ -84,6 +93,12 @@ class AttentionSpec:
     # (a "source" layer may hold that tensor too; it is not read)
     value_mix: str = ""
     value_mix_name: str = "vmix"
+    # q and k of every head pass an RMS norm over the head with a weight [head_dim] that all heads share and this eps,
+    # before the rotation; the weights are named as the q and k matrices plus ``head_norm_suffix``
+    head_norm_eps: float | None = None
+    head_norm_suffix: str = ".norm"
+    # the key projection's raw output (bias added, no norm, no rotation) serves as the values too; the layer has no value matrix
+    value_is_key: bool = False
 
     @property
     def v_dim(self) -> int:
@@ -92,7 +107,8 @@ class AttentionSpec:
     @property
     def general(self) -> bool:
         return bool(self.value_dim not in (0, self.head_dim) or self.qk_norm_eps is not None or self.score_cap or self.chunk or self.sink
-                    or not self.own_kv or self.bias or self.whole_norm_eps is not None or self.slope_exp or self.value_mix)
+                    or not self.own_kv or self.bias or self.whole_norm_eps is not None or self.slope_exp or self.value_mix
+                    or self.head_norm_eps is not None or self.value_is_key)
 
 
 @dataclass(frozen=True)
@@ -138,6 +154,88 @@ class ChannelDeltaSpec:
     norm_eps: float
     decay_rank: int | None = None
     gate_rank: int | None = None
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """A matrix memory with exponential gates (the mLSTM of xLSTM).  With h the input, per head: q = W_q h key_dim^(-1/2),
+    k = W_k h [key_dim], v = W_v h [value_dim], and two gates in the logarithm, i = cap tanh((W_i h + b_i) / cap) and
+    f = logsigmoid(cap tanh((W_f h + b_f) / cap)).  S [key_dim, value_dim], n [key_dim] and a running maximum m start at zero:
+        m' = max(f + m, i);  S <- exp(f + m - m') S + exp(i - m') k v^T;  n likewise with k alone;
+        o = S^T q / (max(|n . q|, exp(-m')) + den_eps)
+    then o / rms(o) per head (``norm_eps``) times a weight over all heads' channels, times sigmoid(W_g h), through W_o.
+    Gates, state and read-out are 32-bit.  ``names``: q, k, v, the output gate, o, the norm weight, the two gate
+    projections (their biases are these names plus ``bias_suffix``), after the prefix."""
+
+    kind: ClassVar[str] = "matrix_memory"
+    hidden: int
+    heads: int
+    key_dim: int
+    value_dim: int
+    gate_cap: float
+    norm_eps: float
+    den_eps: float = 1e-6
+    names: tuple = ("q", "k", "v", "g", "o", "norm", "i", "f")
+    bias_suffix: str = ".b"
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Two mixers side by side that read the same input: left_scale * left(h) + right_scale * right(h).  Each keeps what it
+    keeps (pages, state); their tensors lie under the two prefixes."""
+
+    kind: ClassVar[str] = "parallel"
+    left: object
+    right: object
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    prefixes: tuple[str, str] = ("left.", "right.")
+
+
+@dataclass(frozen=True)
+class ClippedGLUSpec:
+    """One gated feed-forward with clipped inputs: g = min(W_gate h, limit); u = clamp(W_up h, -limit, limit);
+    W_down (g sigmoid(alpha g) (u + 1)).  No biases."""
+
+    intermediate: int
+    limit: float
+    alpha: float = 1.702
+
+
+@dataclass(frozen=True)
+class MoESpec:
+    """A mixture of ``experts`` clipped-GLU feed-forwards of which each token uses ``top``: router logits z = W_r h + b in
+    32-bit, the ``top`` largest are chosen and weighted by the soft-max over the chosen logits alone; ``shared`` (or None)
+    is one more expert that every token uses with weight 1.  Tensor names after the prefix: ``expert_prefix`` + index + "."
+    + gate / up / down, ``router`` and its bias, ``shared_prefix`` + gate / up / down."""
+
+    kind: ClassVar[str] = "moe"
+    hidden: int
+    experts: int
+    top: int
+    expert: ClippedGLUSpec
+    shared: ClippedGLUSpec | None = None
+    names: tuple[str, str, str] = ("gate", "up", "down")
+    expert_prefix: str = "e"
+    router_name: str = "router"
+    router_bias_name: str = "router.b"
+    shared_prefix: str = "shared."
+
+
+@dataclass(frozen=True)
+class TokenSideSpec:
+    """A per-layer input chosen by the token: e = table[token][offset : offset + dim] of a table [vocab, table_dim] that the
+    layers share; y = W_proj (gelu_tanh(W_gate x) * e).  ``table_name`` is the whole tensor name of the table; ``names``: the
+    gate and the projection after the prefix."""
+
+    kind: ClassVar[str] = "token_side"
+    hidden: int
+    vocab: int
+    dim: int
+    offset: int
+    table_dim: int
+    table_name: str = "side.embed"
+    names: tuple[str, str] = ("gate", "proj")
 
 
 @dataclass(frozen=True)
@@ -190,7 +288,9 @@ class StreamBlockSpec:
         u = sum_s in_q[s] x_s;  y = sublayer(norm_q(u));  x_t <- sum_s mix_q[s, t] x_s + mult * out_q[t] * y   (all t at once)
     with the tensors ``prefix + hc_names[q] + "in" | "out" | "mix"``.  ``streams`` = 0: one stream and no such tensors,
     x <- x + mult * sublayer(norm(x)).  ``mixer_post_norm`` / ``ffn_post_norm`` (norm specs or None): a second norm behind
-    the sublayer, y = post_norm(sublayer(norm(u))), in 32-bit on the way into the streams."""
+    the sublayer, y = post_norm(sublayer(norm(u))), in 32-bit on the way into the streams.  A norm in front may be a
+    ``NoNormSpec``: the sublayer then reads u itself.  ``extra`` (or None): a third sublayer behind the feed-forward, a part
+    of the "ffn" role with a norm in front (``extra_norm``) and optionally behind (``extra_post_norm``)."""
 
     kind: ClassVar[str] = "streams"
     prefix: str
@@ -209,6 +309,12 @@ class StreamBlockSpec:
     ffn_post_norm: object | None = None
     mixer_post_norm_name: str = "norm1b"
     ffn_post_norm_name: str = "norm2b"
+    extra: object | None = None
+    extra_norm: object | None = None
+    extra_post_norm: object | None = None
+    extra_prefix: str = "side."
+    extra_norm_name: str = "norm3"
+    extra_post_norm_name: str = "norm3b"
 
 
 @dataclass(frozen=True)

@@ -13,6 +13,7 @@
 // Query head h reads key/value head h / (heads / kv_heads).    (reference: model/attention.py:33)
 // K pages: [page][kv head][token][hd];  V pages: [page][kv head][vd][token].
 #include "common.h"
+#include "rope.h"
 
 #define AG_THREADS 256
 #define AG_MAX_VD 1024  // the largest value size (a thread holds up to four channels of the output)
@@ -236,6 +237,92 @@ extern "C" int ns_whole_norm_kv_write(void* qkv, int stride, const void* bias, c
     whole_norm_kv_write_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((bf16_t*)qkv, stride, (const bf16_t*)bias, (const bf16_t*)qw, (const bf16_t*)kw,
         (const bf16_t*)lambda, (const bf16_t*)v_other, v_other_stride, (bf16_t*)v_keep, v_keep_stride, positions, token_req, block_table,
         table_stride, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, vd, page_size, eps);
+  else
+    return NS_ERR_UNSUPPORTED;
+  return ns_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// Queries and keys with biases, an RMS norm per head whose weight [hd] all heads share, and a rotation of the head's first
+// ``rot`` channels; optionally the key projection's raw output (bias added, no norm, no rotation) is stored as the values.
+// One workgroup a token, a wave a head in turn.  A row of ``qkv`` is [q heads | k heads | v heads] (no v part if
+// ``v_is_k``); q is normed and rotated in place, k and v go into the token's slot of their pages.  All of it in 32-bit.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_rope_kv_write_kernel(
+    T* __restrict__ qkv, int stride, const T* __restrict__ bias, const T* __restrict__ qw, const T* __restrict__ kw,
+    const int* __restrict__ positions, const int* __restrict__ token_req, const int* __restrict__ block_table, int table_stride,
+    const float* __restrict__ inv_freq, T* __restrict__ k_cache, T* __restrict__ v_cache, int heads, int kv_heads, int hd, int vd,
+    int page_size, float eps, RopeForm form, int v_is_k) {
+  const int t = blockIdx.x, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE, waves = blockDim.x / NS_WAVE;
+  T* row = qkv + (size_t)t * stride;
+  const int pos = positions[t];
+  const int page = block_table[(size_t)token_req[t] * table_stride + pos / page_size];
+  const int slot = pos % page_size;
+  const int half = form.rot / 2;
+  for (int h = wave; h < heads + kv_heads; h += waves) {
+    const bool is_q = h < heads;
+    const int at = h * hd;  // q heads and k heads follow each other in the row
+    const T* w = is_q ? qw : kw;
+    float ss = 0.f;
+    for (int c = lane; c < hd; c += NS_WAVE) {
+      const float v = to_f(row[at + c]) + (bias ? to_f(bias[at + c]) : 0.f);
+      ss = fmaf(v, v, ss);
+    }
+    const float rinv = w ? 1.f / sqrtf(wave_sum(ss) / (float)hd + eps) : 1.f;
+    T* kd = is_q ? nullptr : k_cache + (((size_t)page * kv_heads + (h - heads)) * page_size + slot) * hd;
+    if (!is_q && v_is_k) {
+      T* vdst = v_cache + (((size_t)page * kv_heads + (h - heads)) * vd) * page_size + slot;
+      for (int c = lane; c < hd; c += NS_WAVE)
+        vdst[(size_t)c * page_size] = from_f<T>(to_f(row[at + c]) + (bias ? to_f(bias[at + c]) : 0.f));
+    }
+    // the rotated pairs: a lane reads both channels of its pair and writes both
+    for (int j = lane; j < half; j += NS_WAVE) {
+      int d1, d2;
+      rope_pair_channels(form, j, d1, d2);
+      float a = (to_f(row[at + d1]) + (bias ? to_f(bias[at + d1]) : 0.f)) * rinv * (w ? to_f(w[d1]) : 1.f);
+      float b = (to_f(row[at + d2]) + (bias ? to_f(bias[at + d2]) : 0.f)) * rinv * (w ? to_f(w[d2]) : 1.f);
+      float c, s;
+      rope_cos_sin(form, pos, inv_freq[j], c, s);
+      rope_turn(a, b, c, s, a, b);
+      if (is_q) {
+        row[at + d1] = from_f<T>(a);
+        row[at + d2] = from_f<T>(b);
+      } else {
+        kd[d1] = from_f<T>(a);
+        kd[d2] = from_f<T>(b);
+      }
+    }
+    for (int c = form.rot + lane; c < hd; c += NS_WAVE) {
+      const float v = (to_f(row[at + c]) + (bias ? to_f(bias[at + c]) : 0.f)) * rinv * (w ? to_f(w[c]) : 1.f);
+      if (is_q)
+        row[at + c] = from_f<T>(v);
+      else
+        kd[c] = from_f<T>(v);
+    }
+  }
+  if (!v_is_k) {
+    const int nq = heads * hd, nk = kv_heads * hd, nv = kv_heads * vd;
+    for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+      const float v = to_f(row[nq + nk + i]) + (bias ? to_f(bias[nq + nk + i]) : 0.f);
+      v_cache[(((size_t)page * kv_heads + i / vd) * vd + i % vd) * page_size + slot] = from_f<T>(v);
+    }
+  }
+}
+
+extern "C" int ns_head_norm_rope_kv_write(void* qkv, int stride, const void* bias, const void* qw, const void* kw, const int* positions,
+                                          const int* token_req, const int* block_table, int table_stride, const float* inv_freq,
+                                          void* k_cache, void* v_cache, int n_tokens, int heads, int kv_heads, int hd, int vd, int page_size,
+                                          float eps, int rot, int interleaved, float factor, int v_is_k, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || hd <= 0 || vd <= 0 || page_size <= 0 || rot < 0 || rot > hd || rot % 2) return NS_ERR_BAD_ARG;
+  if (v_is_k && vd != hd) return NS_ERR_BAD_ARG;
+  if (rot > 0 && !inv_freq) return NS_ERR_BAD_ARG;
+  const RopeForm form{rot, interleaved, factor};
+  if (dtype == NS_DTYPE_F32)
+    head_norm_rope_kv_write_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, stride, (const float*)bias, (const float*)qw, (const float*)kw,
+        positions, token_req, block_table, table_stride, inv_freq, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, vd, page_size, eps, form, v_is_k);
+  else if (dtype == NS_DTYPE_BF16)
+    head_norm_rope_kv_write_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((bf16_t*)qkv, stride, (const bf16_t*)bias, (const bf16_t*)qw, (const bf16_t*)kw,
+        positions, token_req, block_table, table_stride, inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, vd, page_size, eps, form, v_is_k);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();

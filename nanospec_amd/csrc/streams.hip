@@ -1,7 +1,8 @@
 // A residual stream that is kept in 32-bit whatever the model computes in, and that may be several parallel streams
 // (hyper-connections): x [tokens][S][W], float.  A sublayer reads one mix of the streams through an RMS norm and
 // writes its output back into all of them while the streams are mixed among themselves:
-//   read:   u = sum_s a[s] x_s;            h = w * u / sqrt(mean(u^2) + eps)      (h in the model's precision)
+//   read:   u = sum_s a[s] x_s;            h = w * u / sqrt(mean(u^2) + eps)      (h in the model's precision; without a
+//                                                                                   weight h = u: the sublayer reads the stream itself)
 //   write:  x_t <- sum_s M[s][t] x_s + c[t] y     for all t at once, from the old streams
 // S = 1 with a = M = 1 is the plain pre-norm residual x <- x + c y with its sum in 32-bit.
 // Two options on either side.  A norm's stored weight may be the factor minus one: the factor is then ``w_offset`` + w with
@@ -117,12 +118,12 @@ __global__ void stream_read_norm_kernel(T* __restrict__ out, float* __restrict__
     ss = fmaf(u, u, ss);
   }
   ss = block_sum(ss, scratch);
-  const float rinv = 1.f / sqrtf(ss / (float)W + eps);
+  const float rinv = w ? 1.f / sqrtf(ss / (float)W + eps) : 1.f;  // no weight: no norm, the mix itself is read
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float u = 0.f;
     for (int s = 0; s < S; ++s) u = fmaf(a[s], xr[(size_t)s * W + c], u);
     if (sum_out) sum_out[(size_t)i * W + c] = u;
-    if (out) out[(size_t)i * W + c] = from_f<T>(u * rinv * (w_offset + to_f(w[c])));
+    if (out) out[(size_t)i * W + c] = from_f<T>(w ? u * rinv * (w_offset + to_f(w[c])) : u);
   }
 }
 
@@ -310,17 +311,20 @@ __global__ __launch_bounds__(256) void stream_step_kernel(float* __restrict__ x,
     }
   }
   if (!coeff) return;
-  ss = block_sum(ss, scratch);
-  const float rinv = 1.f / sqrtf(ss / (float)W + eps);
+  if (w) ss = block_sum(ss, scratch);
+  const float rinv = w ? 1.f / sqrtf(ss / (float)W + eps) : 1.f;  // no weight: no norm, the mix itself is read
 #pragma unroll
   for (int k = 0; k < KMAX; ++k) {
     const int c = (threadIdx.x + k * 256) * 4;
     if (c < W) {
       if (sum_out) *reinterpret_cast<float4*>(sum_out + (size_t)i * W + c) = u[k];
-      if (out) {
+      if (out && w) {
         T* op = out + (size_t)i * W + c;
         op[0] = from_f<T>(u[k].x * rinv * (w_offset + to_f(w[c]))), op[1] = from_f<T>(u[k].y * rinv * (w_offset + to_f(w[c + 1])));
         op[2] = from_f<T>(u[k].z * rinv * (w_offset + to_f(w[c + 2]))), op[3] = from_f<T>(u[k].w * rinv * (w_offset + to_f(w[c + 3])));
+      } else if (out) {
+        T* op = out + (size_t)i * W + c;
+        op[0] = from_f<T>(u[k].x), op[1] = from_f<T>(u[k].y), op[2] = from_f<T>(u[k].z), op[3] = from_f<T>(u[k].w);
       }
     }
   }

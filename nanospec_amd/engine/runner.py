@@ -21,6 +21,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage
 from ..kernels import ops
+from ..parts.needs import each_need
 from .arena import Arena
 from .context import BatchLayout, StepContext, fill_batch
 
@@ -101,7 +102,7 @@ class ModelRunner:
         # before the first step on this one
         self.stream.wait_stream(torch.cuda.current_stream(self.device))
         self.arena = Arena(self.device)
-        self._kv_layers = sum(1 for need in model.cache_needs if need is not None and hasattr(need, "kv_heads"))
+        self._kv_layers = sum(1 for need in model.cache_needs for single in each_need(need) if hasattr(single, "kv_heads"))
         self.plans = model.batch_plans() if hasattr(model, "batch_plans") else []  # what the parts want of every batch
         self.link_norms = True  # see StepContext; set False before the first step to run every norm as a kernel of its own
         n_groups = len(manager.groups)

@@ -839,26 +839,34 @@ def embed_streams(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, sca
     return out
 
 
-def stream_read_norm(x: torch.Tensor, coeff: torch.Tensor, weight: torch.Tensor, eps: float, rows: torch.Tensor | None = None,
-                     out: torch.Tensor | None = None, sum_out: torch.Tensor | None = None, w_offset: float = 0.0) -> torch.Tensor:
+def stream_read_norm(x: torch.Tensor, coeff: torch.Tensor, weight: torch.Tensor | None, eps: float, rows: torch.Tensor | None = None,
+                     out: torch.Tensor | None = None, sum_out: torch.Tensor | None = None, w_offset: float = 0.0,
+                     dtype: torch.dtype | None = None) -> torch.Tensor:
     """u = sum_s coeff[s] x[r, s, :] with r = rows[i] (or i); out[i] = (w_offset + weight) * u / sqrt(mean(u^2) + eps) in the weight's dtype.
-    ``x`` float32 [tokens, S, W]; ``sum_out`` (float32 [n, W], optional) also receives u."""
+    ``x`` float32 [tokens, S, W]; ``sum_out`` (float32 [n, W], optional) also receives u.  Without a ``weight`` there is no
+    norm: out[i] = u in ``dtype``."""
     _f32(x, "x"), _f32(coeff, "coeff")
     _gpu(weight, rows, out, sum_out)
-    if x.dim() != 3 or coeff.numel() != x.shape[1] or x.shape[1] > MAX_STREAMS or weight.shape != (x.shape[2],) or not weight.is_contiguous():
+    if weight is None:
+        if dtype is None:
+            raise KernelRefused("stream_read_norm: a read without a norm says in which dtype it wants the stream")
+        weight_dtype = dtype
+    else:
+        weight_dtype = weight.dtype
+    if x.dim() != 3 or coeff.numel() != x.shape[1] or x.shape[1] > MAX_STREAMS or (weight is not None and (weight.shape != (x.shape[2],) or not weight.is_contiguous())):
         raise KernelRefused("stream_read_norm: x is [tokens, S, W], coeff [S], weight [W]")
     if rows is not None:
         _i32(rows, "rows")
     n = rows.numel() if rows is not None else x.shape[0]
     S, W = x.shape[1], x.shape[2]
     if out is None:
-        out = torch.empty((n, W), dtype=weight.dtype, device=x.device)
-    if out.shape != (n, W) or out.dtype != weight.dtype or not out.is_contiguous():
+        out = torch.empty((n, W), dtype=weight_dtype, device=x.device)
+    if out.shape != (n, W) or out.dtype != weight_dtype or not out.is_contiguous():
         raise KernelRefused("stream_read_norm: out must be contiguous [rows, W] of the weight's dtype")
     if sum_out is not None and (_f32(sum_out, "sum_out").shape != (n, W)):
         raise KernelRefused("stream_read_norm: sum_out must be float32 [rows, W]")
     _check(build.core().ns_stream_read_norm(_ptr(out), _ptr(sum_out), _ptr(x), _ptr(coeff), _ptr(weight), _ptr(rows), c_int(n), c_int(S),
-                                            c_int(W), c_float(eps), c_float(w_offset), c_int(_dtype_code(weight)), _stream()), "stream_read_norm")
+                                            c_int(W), c_float(eps), c_float(w_offset), c_int(_dtype_code(out)), _stream()), "stream_read_norm")
     return out
 
 
@@ -916,10 +924,11 @@ class PendingWrite:
 
 def stream_step(x: torch.Tensor, pending: "PendingWrite | None", coeff: torch.Tensor | None = None, weight: torch.Tensor | None = None,
                 eps: float = 0.0, rows: torch.Tensor | None = None, out: torch.Tensor | None = None, sum_out: torch.Tensor | None = None,
-                store: bool = True, w_offset: float = 0.0) -> torch.Tensor | None:
+                store: bool = True, w_offset: float = 0.0, dtype: torch.dtype | None = None) -> torch.Tensor | None:
     """``stream_write`` of ``pending`` (if any) and then ``stream_read_norm`` with ``coeff`` and ``weight`` (if any), in one
     pass over the rows where the sizes allow it, in two kernels otherwise.  With ``rows`` the read is of those rows only,
-    and a pending write is then done on the fly for them and not kept (``store`` must be False): for the last read of a step."""
+    and a pending write is then done on the fly for them and not kept (``store`` must be False): for the last read of a step.
+    A read with ``coeff`` but without ``weight`` has no norm: it gives the mix itself in ``dtype``."""
     S, W = x.shape[1], x.shape[2]
     if pending is not None and rows is not None and store:
         raise KernelRefused("stream_step: a write that is kept covers every row")
@@ -927,7 +936,7 @@ def stream_step(x: torch.Tensor, pending: "PendingWrite | None", coeff: torch.Te
     if not one_pass:
         if pending is not None:  # (kept whatever ``store`` says: keeping it harms nobody)
             stream_write(x, pending.mix, pending.gain, pending.y, pending.post)
-        return stream_read_norm(x, coeff, weight, eps, rows=rows, out=out, sum_out=sum_out, w_offset=w_offset) if coeff is not None else None
+        return stream_read_norm(x, coeff, weight, eps, rows=rows, out=out, sum_out=sum_out, w_offset=w_offset, dtype=dtype) if coeff is not None else None
     _f32(x, "x")
     y = None
     if pending is not None:
@@ -936,12 +945,14 @@ def stream_step(x: torch.Tensor, pending: "PendingWrite | None", coeff: torch.Te
         _gpu(y)
         if pending.mix.shape != (S, S) or pending.gain.shape != (S,) or y.dim() != 2 or y.shape != (x.shape[0], W) or y.stride(1) != 1:
             raise KernelRefused("stream_step: mix [S, S], gain [S], y [tokens, W]")
-    dtype = y.dtype if y is not None else weight.dtype
+    if y is None and weight is None and coeff is not None and dtype is None:
+        raise KernelRefused("stream_step: a read without a norm says in which dtype it wants the stream")
+    dtype = y.dtype if y is not None else (weight.dtype if weight is not None else dtype)
     n = x.shape[0]
     if coeff is not None:
         _f32(coeff, "coeff")
         _gpu(weight, rows, out, sum_out)
-        if coeff.numel() != S or weight.shape != (W,) or not weight.is_contiguous() or weight.dtype != dtype:
+        if coeff.numel() != S or (weight is not None and (weight.shape != (W,) or not weight.is_contiguous() or weight.dtype != dtype)):
             raise KernelRefused("stream_step: coeff [S], weight [W] in the dtype of y")
         if rows is not None:
             _i32(rows, "rows")
@@ -1020,6 +1031,191 @@ def whole_norm_kv_write(qkv: torch.Tensor, positions, token_req, block_table, k_
                                                _ptr(block_table), c_int(block_table.stride(0)), _ptr(k_cache), _ptr(v_cache), c_int(n),
                                                c_int(heads), c_int(kv_heads), c_int(head_dim), c_int(v_dim), c_int(page), c_float(eps),
                                                c_int(_dtype_code(qkv)), _stream()), "whole_norm_kv_write")
+
+
+def head_norm_rope_kv_write(qkv: torch.Tensor, positions, token_req, block_table, inv_freq, k_cache, v_cache, heads: int, kv_heads: int,
+                            head_dim: int, v_dim: int, eps: float, rotary_dim: int, bias: torch.Tensor | None = None,
+                            q_weight: torch.Tensor | None = None, k_weight: torch.Tensor | None = None, value_is_key: bool = False,
+                            interleaved: bool = False, factor: float = 1.0) -> None:
+    """For attention whose queries and keys pass an RMS norm per head and then a rotation.  A row of ``qkv`` is q [heads *
+    head_dim], k [kv_heads * head_dim] and, unless ``value_is_key``, v [kv_heads * v_dim]; ``bias`` of that width is added.
+    q (in place) and k become x / sqrt(mean(x^2 over the head) + eps) * weight (``q_weight``, ``k_weight`` [head_dim], shared
+    by the heads; None: no norm), then their first ``rotary_dim`` channels are rotated by the token's position.  With
+    ``value_is_key`` the key projection's raw output (bias added, ahead of norm and rotation) is stored as the values.  k and v go into the
+    pages of their positions."""
+    _gpu(qkv, positions, token_req, block_table, k_cache, v_cache, bias, q_weight, k_weight, inv_freq)
+    n = positions.numel()
+    nq, nk, nv = heads * head_dim, kv_heads * head_dim, 0 if value_is_key else kv_heads * v_dim
+    if qkv.dim() != 2 or qkv.shape[0] != n or qkv.shape[1] < nq + nk + nv or qkv.stride(1) != 1:
+        raise KernelRefused(f"head_norm_rope_kv_write: qkv must be [{n}, {nq + nk + nv}]")
+    if value_is_key and v_dim != head_dim:
+        raise KernelRefused("head_norm_rope_kv_write: values that are the keys have the keys' size")
+    _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
+    if token_req.numel() != n or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelRefused("head_norm_rope_kv_write: token_req is per token, block_table int32 [requests, pages]")
+    page = k_cache.shape[2] if k_cache.dim() == 4 else 0
+    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, v_dim, page)
+            or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+        raise KernelRefused("head_norm_rope_kv_write: cache pages do not fit heads, sizes or dtype")
+    for t, size, name in ((bias, nq + nk + nv, "bias"), (q_weight, head_dim, "q_weight"), (k_weight, head_dim, "k_weight")):
+        if t is not None and (t.numel() != size or not t.is_contiguous() or t.dtype != qkv.dtype):
+            raise KernelRefused(f"head_norm_rope_kv_write: {name} holds {size} values of the dtype of qkv")
+    if rotary_dim % 2 or not 0 <= rotary_dim <= head_dim:
+        raise KernelRefused("head_norm_rope_kv_write: the rotated channels of a head are an even number, at most the head")
+    if rotary_dim and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2 or not inv_freq.is_contiguous()):
+        raise KernelRefused("head_norm_rope_kv_write: inv_freq is float32 [rotary_dim / 2]")
+    _check(build.core().ns_head_norm_rope_kv_write(_ptr(qkv), c_int(qkv.stride(0)), _ptr(bias), _ptr(q_weight), _ptr(k_weight), _ptr(positions),
+                                                   _ptr(token_req), _ptr(block_table), c_int(block_table.stride(0)), _ptr(inv_freq),
+                                                   _ptr(k_cache), _ptr(v_cache), c_int(n), c_int(heads), c_int(kv_heads), c_int(head_dim),
+                                                   c_int(v_dim), c_int(page), c_float(eps), c_int(rotary_dim), c_int(1 if interleaved else 0),
+                                                   c_float(factor), c_int(1 if value_is_key else 0), c_int(_dtype_code(qkv)), _stream()),
+           "head_norm_rope_kv_write")
+
+
+# ------------------------------------------------------------------------------------------------ matrix memory
+
+
+MEMORY_MAX_KEY_DIM = 512  # key channels of a head that ``memory_scan`` takes (a column's channels are 8 to a lane of one wave)
+MOE_MAX_EXPERTS, MOE_MAX_TOP = 1024, 32
+
+
+def memory_blocks(key_dim: int, value_dim: int) -> int:
+    """Workgroups that share the columns of one head in ``memory_scan``: the state keeps a copy of n and m for each."""
+    b = int(build.core().ns_memory_blocks(c_int(key_dim), c_int(value_dim)))
+    if b < 0:
+        raise KernelRefused(f"memory_scan takes key sizes up to 512, not {key_dim}")
+    return b
+
+
+def memory_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
+    """32-bit words of a request's state: S [heads, value_dim, key_dim], then n [heads, blocks, key_dim] and m [heads, blocks]."""
+    return heads * value_dim * key_dim + heads * memory_blocks(key_dim, value_dim) * (key_dim + 1)
+
+
+def memory_scan(proj: torch.Tensor, offsets: tuple[int, int, int, int, int], gate_bias_i: torch.Tensor | None, gate_bias_f: torch.Tensor | None,
+                state: torch.Tensor, qo_indptr, state_slots, heads: int, key_dim: int, value_dim: int, cap: float, q_scale: float,
+                out: torch.Tensor, den_eps: float = 1e-6) -> torch.Tensor:
+    """The matrix memory's recurrence over every request's tokens of the step, in order (``csrc/memory.hip``).  A row of
+    ``proj`` holds q and k [heads * key_dim], v [heads * value_dim] and the two gate inputs [heads] at the column
+    ``offsets`` (q, k, v, input gate, forget gate); ``state`` float32 [slots, >= memory_state_floats]; ``out`` float32
+    [tokens, heads * value_dim]."""
+    _gpu(proj, state, qo_indptr, state_slots, out, gate_bias_i, gate_bias_f)
+    _f32(out, "out"), _i32(qo_indptr, "qo_indptr"), _i32(state_slots, "state_slots")
+    n = proj.shape[0]
+    q_off, k_off, v_off, i_off, f_off = offsets
+    if proj.dim() != 2 or proj.stride(1) != 1 or max(q_off, k_off) + heads * key_dim > proj.shape[1] or v_off + heads * value_dim > proj.shape[1] \
+            or max(i_off, f_off) + heads > proj.shape[1]:
+        raise KernelRefused("memory_scan: the row does not hold q, k, v and the gates at the given columns")
+    if out.shape != (n, heads * value_dim):
+        raise KernelRefused(f"memory_scan: out must be float32 [{n}, {heads * value_dim}]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < memory_state_floats(heads, key_dim, value_dim):
+        raise KernelRefused("memory_scan: state is float32 [slots, words] with room for S, n and m")
+    for t in (gate_bias_i, gate_bias_f):
+        if t is not None and (_f32(t, "gate bias").numel() != heads):
+            raise KernelRefused("memory_scan: a gate's bias is float32 [heads]")
+    reqs = qo_indptr.numel() - 1
+    if state_slots.numel() < reqs:
+        raise KernelRefused("memory_scan: one state slot per request")
+    _check(build.core().ns_memory_scan(_ptr(proj), c_int(proj.stride(0)), c_int(q_off), c_int(k_off), c_int(v_off), c_int(i_off), c_int(f_off),
+                                       _ptr(gate_bias_i), _ptr(gate_bias_f), _ptr(state), ctypes.c_longlong(state.stride(0)), _ptr(qo_indptr),
+                                       _ptr(state_slots), _ptr(out), c_int(reqs), c_int(heads), c_int(key_dim), c_int(value_dim), c_float(cap),
+                                       c_float(q_scale), c_float(den_eps), c_int(_dtype_code(proj)), _stream()), "memory_scan")
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ mixture of experts
+
+
+def moe_route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, top: int, sel: torch.Tensor, weights: torch.Tensor) -> None:
+    """Router logits z = router h + bias in 32-bit (``router`` float32 [experts, W]); ``sel`` int32 [tokens, top] receives the
+    experts with the largest logits in falling order, ``weights`` float32 [tokens, top] the soft-max over those logits."""
+    _gpu(h, router, bias, sel, weights)
+    _f32(router, "router"), _f32(weights, "weights"), _i32(sel, "sel")
+    n, W = h.shape
+    experts = router.shape[0]
+    if h.stride(1) != 1 or router.shape != (experts, W) or sel.shape != (n, top) or weights.shape != (n, top) or (bias is not None and _f32(bias, "bias").numel() != experts):
+        raise KernelRefused("moe_route: h [tokens, W], router [experts, W], bias [experts], sel and weights [tokens, top]")
+    _check(build.core().ns_moe_route(_ptr(h), c_int(h.stride(0)), _ptr(router), _ptr(bias), _ptr(sel), _ptr(weights), c_int(n), c_int(W),
+                                     c_int(experts), c_int(top), c_int(_dtype_code(h)), _stream()), "moe_route")
+
+
+def moe_expert_rows(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
+                    limit: float, alpha: float, out: torch.Tensor) -> torch.Tensor:
+    """out[t, k] = weights[t, k] * expert sel[t, k] of h[t]: one workgroup per (token, chosen expert).  ``gate``, ``up``
+    [experts, ff, W], ``down`` [experts, W, ff] in the dtype of ``h``; ``out`` float32 [tokens, top, W]."""
+    _gpu(h, gate, up, down, sel, weights, out)
+    _f32(out, "out"), _f32(weights, "weights"), _i32(sel, "sel")
+    n, W = h.shape
+    experts, ff = gate.shape[0], gate.shape[1]
+    top = sel.shape[1]
+    if (h.stride(1) != 1 or gate.shape != (experts, ff, W) or up.shape != gate.shape or down.shape != (experts, W, ff) or sel.shape != (n, top)
+            or weights.shape != (n, top) or out.shape != (n, top, W) or any(t.dtype != h.dtype or not t.is_contiguous() for t in (gate, up, down))):
+        raise KernelRefused("moe_expert_rows: gate and up [experts, ff, W], down [experts, W, ff] in the dtype of h; out float32 [tokens, top, W]")
+    _check(build.core().ns_moe_expert_rows(_ptr(h), c_int(h.stride(0)), _ptr(gate), _ptr(up), _ptr(down), _ptr(sel), _ptr(weights), _ptr(out),
+                                           c_int(n), c_int(W), c_int(ff), c_int(top), c_float(limit), c_float(alpha), c_int(_dtype_code(h)),
+                                           _stream()), "moe_expert_rows")
+    return out
+
+
+def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
+                limit: float, alpha: float, take) -> torch.Tensor:
+    """The chosen experts' weighted outputs, float32 [tokens, top, W], by the kernel that suits the number of rows.
+    ``take(shape, dtype)`` gives scratch that lives as long as the result."""
+    n, W = h.shape
+    top = sel.shape[1]
+    return moe_expert_rows(h, gate, up, down, sel, weights, limit, alpha, take((n, top, W), torch.float32))
+
+
+def clipped_glu(gu: torch.Tensor, limit: float, alpha: float, out: torch.Tensor) -> torch.Tensor:
+    """out = g sigmoid(alpha g) (u + 1) with g = min(gu[:, :ff], limit), u = clamp(gu[:, ff:], -limit, limit)."""
+    _gpu(gu, out)
+    n, ff = out.shape
+    if gu.shape != (n, 2 * ff) or gu.stride(1) != 1 or not out.is_contiguous() or out.dtype != gu.dtype:
+        raise KernelRefused("clipped_glu: gu [tokens, 2 ff], out [tokens, ff] of the same dtype")
+    _check(build.core().ns_clipped_glu(_ptr(out), _ptr(gu), c_int(gu.stride(0)), c_int(n), c_int(ff), c_float(limit), c_float(alpha),
+                                       c_int(_dtype_code(gu)), _stream()), "clipped_glu")
+    return out
+
+
+def moe_combine(parts: torch.Tensor, base: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = base[t] + sum_k parts[t, k] (``parts`` float32 [tokens, top, W]; ``base`` and ``out`` in the model's dtype)."""
+    _gpu(parts, base, out)
+    _f32(parts, "parts")
+    n, top, W = parts.shape
+    if out.shape != (n, W) or not out.is_contiguous() or (base is not None and (base.shape != (n, W) or not base.is_contiguous() or base.dtype != out.dtype)):
+        raise KernelRefused("moe_combine: base and out are contiguous [tokens, W] of one dtype")
+    _check(build.core().ns_moe_combine(_ptr(out), _ptr(base), _ptr(parts), c_int(n), c_int(top), c_int(W), c_int(_dtype_code(out)), _stream()),
+           "moe_combine")
+    return out
+
+
+def scaled_sum(a: torch.Tensor, b: torch.Tensor, sa: float, sb: float, out: torch.Tensor, bias: torch.Tensor | None = None,
+               bias_b: torch.Tensor | None = None) -> torch.Tensor:
+    """out = sa * (a + bias) + sb * (b + bias_b), formed in 32-bit (the biases [W] or None)."""
+    _gpu(a, b, out, bias, bias_b)
+    n, W = a.shape
+    if any(t.shape != (n, W) or not t.is_contiguous() or t.dtype != a.dtype for t in (b, out)) or not a.is_contiguous():
+        raise KernelRefused("scaled_sum: a, b and out are contiguous [tokens, W] of one dtype")
+    for t in (bias, bias_b):
+        if t is not None and (t.numel() != W or t.dtype != a.dtype or not t.is_contiguous()):
+            raise KernelRefused("scaled_sum: a bias is [W] of the same dtype")
+    _check(build.core().ns_scaled_sum(_ptr(out), _ptr(a), _ptr(b), _ptr(bias), _ptr(bias_b), c_float(sa), c_float(sb), c_int(n), c_int(W),
+                                      c_int(_dtype_code(a)), _stream()), "scaled_sum")
+    return out
+
+
+def token_side(x: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, gate: torch.Tensor, proj: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = proj (gelu_tanh(gate x[t]) * table[ids[t]]): ``table`` [vocab, dim], ``gate`` [dim, W], ``proj`` [W, dim]."""
+    _gpu(x, ids, table, gate, proj, out)
+    _i32(ids, "ids")
+    n, W = x.shape
+    dim = table.shape[1]
+    if (x.stride(1) != 1 or ids.numel() != n or gate.shape != (dim, W) or proj.shape != (W, dim) or out.shape != (n, W) or not out.is_contiguous()
+            or any(t.dtype != x.dtype or not t.is_contiguous() for t in (table, gate, proj)) or out.dtype != x.dtype):
+        raise KernelRefused("token_side: table [vocab, dim], gate [dim, W], proj [W, dim], all in the dtype of x")
+    _check(build.core().ns_token_side(_ptr(out), _ptr(x), c_int(x.stride(0)), _ptr(ids), _ptr(table), _ptr(gate), _ptr(proj), c_int(n), c_int(W),
+                                      c_int(dim), c_int(_dtype_code(x)), _stream()), "token_side")
+    return out
 
 
 def silu_mul_bias(gu: torch.Tensor, bias: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -1225,14 +1421,16 @@ def delta_scan(qkv: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, state: to
 
 def gated_rms(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, out: torch.Tensor) -> torch.Tensor:
     """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight * sigmoid(gate[t, h, :]); ``o`` float32 [tokens,
-    heads * E], ``weight`` float32 [E], ``gate`` (may be a column slice) and ``out`` in the model's dtype."""
+    heads * E], ``weight`` float32 [E] (all heads share it) or [heads * E], ``gate`` (may be a column slice) and ``out`` in the
+    model's dtype."""
     _f32(o, "o"), _f32(weight, "weight")
     _gpu(gate, out)
     n, width = o.shape
-    if (width % heads or weight.numel() != width // heads or gate.shape[0] != n or gate.shape[1] < width or gate.stride(1) != 1
+    if (width % heads or weight.numel() not in (width // heads, width) or gate.shape[0] != n or gate.shape[1] < width or gate.stride(1) != 1
             or out.shape != (n, width) or not out.is_contiguous() or out.dtype != gate.dtype):
         raise KernelRefused("gated_rms: operands do not fit heads and value size")
-    _check(build.core().ns_gated_rms(_ptr(out), _ptr(o), _ptr(gate), c_int(gate.stride(0)), _ptr(weight), c_int(n), c_int(heads),
+    per_head = width // heads if (weight.numel() == width and heads > 1) else 0
+    _check(build.core().ns_gated_rms(_ptr(out), _ptr(o), _ptr(gate), c_int(gate.stride(0)), _ptr(weight), c_int(per_head), c_int(n), c_int(heads),
                                      c_int(width // heads), c_float(eps), c_int(_dtype_code(gate)), _stream()), "gated_rms")
     return out
 

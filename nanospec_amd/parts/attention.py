@@ -197,6 +197,12 @@ class Attention:
             raise ValueError("biases, whole-projection norms and mixed values belong to a layer with key/value projections of its own")
         if spec.whole_norm_eps is not None and (spec.qk_norm_eps is not None or self.position.rotary_dim):
             raise ValueError("a norm over the whole projection stands alone: no per-head unit norm and no rotation beside it")
+        self.head_form = spec.head_norm_eps is not None or spec.value_is_key  # per-head norms with weights, values that are the keys
+        if self.head_form and (spec.qk_norm_eps is not None or spec.whole_norm_eps is not None or spec.value_mix or not spec.own_kv):
+            raise ValueError("per-head norms with weights and values that are the keys stand beside biases and a rotation only")
+        if spec.value_is_key and spec.v_dim != spec.head_dim:
+            raise ValueError("values that are the keys have the keys' size")
+        self.q_head_norm = self.k_head_norm = None
 
     VALUES_KEY = "attention.values"  # where a "source" layer leaves its values of the step's tokens (``ctx.shared``)
 
@@ -216,10 +222,15 @@ class Attention:
         out = {q: ((s.heads * s.head_dim, s.hidden), "linear"), o: ((s.hidden, s.heads * s.v_dim), "linear"), **self.position.wanted()}
         if s.own_kv:
             out[k] = ((s.kv_heads * s.head_dim, s.hidden), "linear")
-            out[v] = ((s.kv_heads * s.v_dim, s.hidden), "linear")
+            if not s.value_is_key:
+                out[v] = ((s.kv_heads * s.v_dim, s.hidden), "linear")
         if s.bias:
             for name in (q, k, v, o):
-                out[name + s.bias_suffix] = ((out[name][0][0],), "bias")
+                if name in out:
+                    out[name + s.bias_suffix] = ((out[name][0][0],), "bias")
+        if s.head_norm_eps is not None:
+            out[q + s.head_norm_suffix] = ((s.head_dim,), "norm")
+            out[k + s.head_norm_suffix] = ((s.head_dim,), "norm")
         if s.whole_norm_eps is not None:
             out[q + s.whole_norm_suffix] = ((s.heads * s.head_dim,), "norm")
             out[k + s.whole_norm_suffix] = ((s.kv_heads * s.head_dim,), "norm")
@@ -233,10 +244,11 @@ class Attention:
         s = self.spec
         plain = layouts == "both"
         q, k, v, o = self._names
-        rows = s.heads * s.head_dim + (s.kv_heads * (s.head_dim + s.v_dim) if s.own_kv else 0)
+        rows = s.heads * s.head_dim + (s.kv_heads * (s.head_dim + (0 if s.value_is_key else s.v_dim)) if s.own_kv else 0)
         wqkv = torch.empty((rows, s.hidden), dtype=dtype, device=device)
         at = 0
-        for name in (q, k, v) if s.own_kv else (q,):
+        stacked = (q,) if not s.own_kv else ((q, k) if s.value_is_key else (q, k, v))
+        for name in stacked:
             t = get(name)
             wqkv[at : at + t.shape[0]].copy_(t)
             at += t.shape[0]
@@ -245,8 +257,10 @@ class Attention:
         self._form = dict(interleaved=bool(getattr(self.position, "interleaved", False)), factor=float(getattr(self.position, "factor", 1.0)))
         to = lambda name: get(name).to(device=device, dtype=dtype).contiguous()
         if s.bias:
-            self.qkv_bias = torch.cat([to(name + s.bias_suffix) for name in (q, k, v)]).contiguous()
+            self.qkv_bias = torch.cat([to(name + s.bias_suffix) for name in stacked]).contiguous()
             self.out_bias = to(o + s.bias_suffix)
+        if s.head_norm_eps is not None:
+            self.q_head_norm, self.k_head_norm = to(q + s.head_norm_suffix), to(k + s.head_norm_suffix)
         if s.whole_norm_eps is not None:
             self.q_norm, self.k_norm = to(q + s.whole_norm_suffix), to(k + s.whole_norm_suffix)
         if s.value_mix == "mix":
@@ -342,7 +356,13 @@ class Attention:
         if cache.k.shape[1:] != (s.kv_heads, cache.k.shape[2], s.head_dim) or cache.v.shape[2] != s.v_dim:
             raise ValueError("the cache that this layer reads has other heads or sizes than the layer")
         self.wqkv(x, out=qkv, arena=ctx.arena, plain_copy=not ctx.captured)
-        if pos.rotary_dim:
+        if self.head_form:
+            if pos.max_positions is not None and ctx.max_position >= pos.max_positions:
+                raise ValueError(f"position {ctx.max_position} is beyond the model's {pos.max_positions} positions")
+            ops.head_norm_rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq if pos.rotary_dim else None, cache.k, cache.v,
+                                        s.heads, s.kv_heads, s.head_dim, s.v_dim, s.head_norm_eps or 0.0, pos.rotary_dim, bias=self.qkv_bias,
+                                        q_weight=self.q_head_norm, k_weight=self.k_head_norm, value_is_key=s.value_is_key, **self._form)
+        elif pos.rotary_dim:
             if s.qk_norm_eps is not None or s.v_dim != s.head_dim or not s.own_kv:
                 raise ops.KernelRefused("rotation together with unit-RMS queries and keys, another value size or borrowed keys is not built")
             if s.bias or s.value_mix:

@@ -129,11 +129,18 @@ class StreamBlock:
         post = lambda given, name: registry.build("norm", given, p + name) if given is not None else None
         self.mixer_post = post(getattr(spec, "mixer_post_norm", None), getattr(spec, "mixer_post_norm_name", ""))
         self.ffn_post = post(getattr(spec, "ffn_post_norm", None), getattr(spec, "ffn_post_norm_name", "")) if spec.ffn is not None else None
-        self.parts = tuple(x for x in (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post) if x is not None)
-        for norm in (self.mixer_norm, self.ffn_norm):
+        # a third sublayer behind the feed-forward (a part of the "ffn" role: it sees the step's context and its input)
+        extra = getattr(spec, "extra", None)
+        self.extra = registry.build("ffn", extra, p + spec.extra_prefix) if extra is not None else None
+        self.extra_norm = registry.build("norm", spec.extra_norm, p + spec.extra_norm_name) if extra is not None else None
+        self.extra_post = post(spec.extra_post_norm, spec.extra_post_norm_name) if extra is not None else None
+        self.parts = tuple(x for x in (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post,
+                                       self.extra_norm, self.extra, self.extra_post) if x is not None)
+        self.dtype = None
+        for norm in (self.mixer_norm, self.ffn_norm, self.extra_norm):
             if norm is not None and not hasattr(norm, "read_streams"):
                 raise ValueError(f"a norm of kind {norm.spec.kind!r} cannot read a 32-bit stream (it has no read_streams)")
-        for norm in (self.mixer_post, self.ffn_post):
+        for norm in (self.mixer_post, self.ffn_post, self.extra_post):
             if norm is not None and not hasattr(norm, "behind"):
                 raise ValueError(f"a norm of kind {norm.spec.kind!r} cannot stand behind a sublayer of a 32-bit stream (it has no behind)")
         self._hc: list = []  # per sublayer: (in [S], mix [S, S], mult * out [S]) float32 on the device
@@ -143,6 +150,8 @@ class StreamBlock:
         return all(getattr(p, "graph_safe", False) for p in self.parts)
 
     def _hc_names(self):
+        if self.extra is not None:
+            raise ValueError("hyper-connected streams with a third sublayer are not built")
         return [self.prefix + q + t for q in self.spec.hc_names[: 2 if self.ffn is not None else 1] for t in ("in", "out", "mix")]
 
     def wanted(self) -> dict:
@@ -171,9 +180,10 @@ class StreamBlock:
             else:
                 p.load(get, dtype, device)
         S, m = self.copies, float(self.spec.mult)
+        self.dtype = dtype
         self._hc = []
         f32 = lambda t: t.to(device=device, dtype=torch.float32).contiguous()
-        for q in range(2 if self.ffn is not None else 1):
+        for q in range(3 if self.extra is not None else (2 if self.ffn is not None else 1)):
             if self.spec.streams:
                 pre = self.prefix + self.spec.hc_names[q]
                 self._hc.append((f32(get(pre + "in")), f32(get(pre + "mix")), f32(get(pre + "out")) * m))
@@ -214,17 +224,19 @@ class StreamBlock:
         if S != self.copies:
             raise ValueError(f"the block is built for {self.copies} streams, the model carries {S}")
         mark = ctx.arena.mark()
-        dtype = self.mixer_norm.weight.dtype
+        dtype = self.dtype
         a, mix, gain = self._hc[0]
         h = self.mixer_norm.read_streams(ctx, resid, a, out=ctx.arena.take((n, W), dtype), pending=delta)
-        last = self.ffn is None
+        later = [(self.ffn_norm, self.ffn, self.ffn_post, 1)] if self.ffn is not None else []
+        if self.extra is not None:
+            later.append((self.extra_norm, self.extra, self.extra_post, 2))
         y, post = self._sublayer(self.mixer, self.mixer_post, ctx, h, cache, owns_cache,
-                                 out=delta_out if last and delta_out is not None else ctx.arena.take((n, W), dtype))
+                                 out=delta_out if not later and delta_out is not None else ctx.arena.take((n, W), dtype))
         pending = ops.PendingWrite(y, mix, gain, post)
-        if not last:
-            a, mix, gain = self._hc[1]
-            h = self.ffn_norm.read_streams(ctx, resid, a, out=h, pending=pending)
-            y, post = self._sublayer(self.ffn, self.ffn_post, ctx, h, out=delta_out if delta_out is not None else y)
+        for at, (norm, part, post_norm, q) in enumerate(later):
+            a, mix, gain = self._hc[q]
+            h = norm.read_streams(ctx, resid, a, out=h, pending=pending)
+            y, post = self._sublayer(part, post_norm, ctx, h, out=delta_out if (delta_out is not None and at == len(later) - 1) else y)
             pending = ops.PendingWrite(y, mix, gain, post)
         if delta_out is None:
             ops.stream_step(resid, pending)

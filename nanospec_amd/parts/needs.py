@@ -1,4 +1,5 @@
-"""What a mixer asks of the cache manager."""
+"""What a mixer asks of the cache manager: pages (``PagedNeed``), state of fixed size (``StateNeed``), nothing (None), or a
+tuple of these for a mixer made of several (it is then handed a tuple of views in the same order)."""
 
 from __future__ import annotations
 
@@ -32,3 +33,12 @@ class StateNeed:
 
     shape: tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+
+def each_need(need):
+    """The single needs of what ``cache_need()`` returned, in order."""
+    if isinstance(need, (tuple, list)):
+        for n in need:
+            yield from each_need(n)
+    elif need is not None:
+        yield need

@@ -49,4 +49,30 @@ class RMSNorm:
         return ops.PostNorm(bias, self.weight, self.spec.eps, self.offset)
 
 
+class NoNorm:
+    """No norm: a sublayer behind it reads the mix of a 32-bit stream's copies itself, rounded to the model's precision."""
+
+    graph_safe = True
+    links_products = False
+    weight = None
+
+    def __init__(self, spec, name: str) -> None:
+        self.spec, self.name = spec, name
+        self.dtype: torch.dtype | None = None
+
+    def wanted(self) -> dict:
+        return {}
+
+    def load(self, get, dtype, device) -> None:
+        self.dtype = dtype
+
+    def forward(self, ctx, resid=None, x=None, rows=None, write_resid=False, out=None) -> torch.Tensor:
+        raise ops.KernelRefused("a read without a norm is built for 32-bit streams (blocks of kind 'streams')")
+
+    def read_streams(self, ctx, streams: torch.Tensor, coeff: torch.Tensor, rows=None, out=None, sum_out=None, pending=None,
+                     store: bool = True) -> torch.Tensor:
+        return ops.stream_step(streams, pending, coeff, None, 0.0, rows=rows, out=out, sum_out=sum_out, store=store, dtype=self.dtype)
+
+
 register("norm", "rmsnorm", RMSNorm)
+register("norm", "none", NoNorm)
