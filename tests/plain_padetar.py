@@ -65,7 +65,8 @@ def left_attention(h: torch.Tensor, w: dict, p: str, m: dict, eps: float, positi
     v = k
     q = rms(q, eps) * w[p + "q.norm"]
     kn = rms(k, eps) * w[p + "k.norm"]
-    q, kn = rotate(q, positions, m["rot"]), rotate(kn, positions, m["rot"])
+    if m.get("rot"):
+        q, kn = rotate(q, positions, m["rot"]), rotate(kn, positions, m["rot"])
     out = torch.zeros(T, H, D, dtype=h.dtype)
     mask = torch.tril(torch.ones(T, T, dtype=torch.bool))
     for a in range(H):
