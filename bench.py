@@ -254,6 +254,26 @@ def fetitar_config(shape: dict, layers: int | None = None):
                                   "embedding": {"scale": 1.0, "bigram": {"buckets": 65536, "mul_prev": 127, "mul_cur": 7}}, "layers": entries})
 
 
+# Sizes for ``--design padetar``: the Padetar design at the widths, depths and head counts of the Llama shapes above.  Every
+# layer's left mixer has the shape's heads and key/value heads (the whole head rotated, Llama-3.1 frequency scaling), its
+# right mixer is a matrix memory of width / 256 heads with 128 key and 256 value channels; the feed-forward is 32 experts of
+# an eighth of the shape's inner size, four of them per token, beside a shared expert of half the inner size (so a token
+# passes as many inner channels as in the Llama model); a token input of 256 columns per layer.
+def padetar_config(shape: dict, layers: int | None = None):
+    from nanospec_amd.config import PadetarConfig
+
+    n = layers or shape["num_hidden_layers"]
+    heads, kvh, hd, ff, width = (shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"], shape["intermediate_size"],
+                                 shape["hidden_size"])
+    left = dict(heads=heads, kv_heads=kvh, dim=hd, vdim=hd, scale=hd ** -0.5,
+                rot={"base": 1e6, "dims": hd, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}})
+    right = dict(heads=width // 256, dim=128, vdim=256, gate_cap=15.0)
+    mlp = {"kind": "moe", "router": {"experts": 32, "top": 4}, "expert": {"ff": ff // 8, "limit": 7.0}, "shared": {"ff": ff // 2, "limit": 7.0}}
+    entry = {"type": "parallel", "mixer": {"left": left, "left_scale": 1.0, "right": right, "right_scale": 1.0}, "mlp": mlp}
+    return PadetarConfig.from_hf({"architecture": "Padetar", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-5},
+                                  "token_side": {"dim": 256}, "layers": [entry] * n})
+
+
 def design_compare(a) -> int:
     """``--design NAME``: prefill and decode throughput of that design beside the Llama model of the same shape,
     one JSON line.  The default workload and its output are not touched by this option."""
@@ -271,7 +291,7 @@ def design_compare(a) -> int:
     llama = LlamaConfig.from_hf(dict(model_type="llama", **{k: v for k, v in shape.items() if k != "rope_scaling"},
                                      rope_scaling=dict(rope_type="llama3", **shape["rope_scaling"])))
     design = a.design
-    vz = vuzelix_config(shape) if design == "vuzelix" else fetitar_config(shape)
+    vz = {"vuzelix": vuzelix_config, "fetitar": fetitar_config, "padetar": padetar_config}[design](shape)
     out = {}
     k = min(a.steps, 128)
     for name, cfg in (("llama", llama), (design, vz)):
@@ -314,7 +334,7 @@ def main() -> int:
                     help="instead of the benchmark: continuous batching of this many requests (prompts of 16 to 1,024 tokens, 128 new "
                          "tokens each, prompts in portions of 512)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="the benchmark's shape is 8b; the others are for profiles")
-    ap.add_argument("--design", default=None, choices=["vuzelix", "fetitar"],
+    ap.add_argument("--design", default=None, choices=["vuzelix", "fetitar", "padetar"],
                     help="instead of the benchmark: prefill and decode of this design beside the Llama model of the same --shape")
     a = ap.parse_args()
     if a.gpus != 1:

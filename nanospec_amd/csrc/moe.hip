@@ -9,23 +9,37 @@
 #define MOE_MAX_EXPERTS 1024
 #define MOE_MAX_TOP 32
 
-// One workgroup a token: every wave takes experts in turn, its lanes share the row; thread 0 then chooses.
+// One workgroup takes ROUTE_TOK tokens: every wave takes experts in turn and reads an expert's row once for all of the
+// tokens; one thread a token then chooses.
+#define ROUTE_TOK 8
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, int h_stride, const float* __restrict__ wr,
                                                         const float* __restrict__ br, int* __restrict__ sel, float* __restrict__ wt,
-                                                        int W, int experts, int top) {
-  __shared__ float z[MOE_MAX_EXPERTS];
-  const int t = blockIdx.x, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE, waves = blockDim.x / NS_WAVE;
-  const T* x = h + (size_t)t * h_stride;
+                                                        int n, int W, int experts, int top) {
+  __shared__ float z[ROUTE_TOK][MOE_MAX_EXPERTS];
+  const int t0 = blockIdx.x * ROUTE_TOK, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE, waves = blockDim.x / NS_WAVE;
+  const int nt = min(ROUTE_TOK, n - t0);
   for (int e = wave; e < experts; e += waves) {
     const float* w = wr + (size_t)e * W;
-    float acc = 0.f;
-    for (int c = lane; c < W; c += NS_WAVE) acc = fmaf(to_f(x[c]), w[c], acc);
-    acc = wave_sum(acc);
-    if (lane == 0) z[e] = acc + (br ? br[e] : 0.f);
+    float acc[ROUTE_TOK];
+#pragma unroll
+    for (int i = 0; i < ROUTE_TOK; ++i) acc[i] = 0.f;
+    for (int c = lane; c < W; c += NS_WAVE) {
+      const float wc = w[c];
+#pragma unroll
+      for (int i = 0; i < ROUTE_TOK; ++i)
+        if (i < nt) acc[i] = fmaf(to_f(h[(size_t)(t0 + i) * h_stride + c]), wc, acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < ROUTE_TOK; ++i) {
+      const float v = wave_sum(acc[i]);
+      if (lane == 0) z[i][e] = v + (br ? br[e] : 0.f);
+    }
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
+  if (threadIdx.x < nt) {
+    const int t = t0 + threadIdx.x;
+    const float* zt = z[threadIdx.x];
     int idx[MOE_MAX_TOP];
     float val[MOE_MAX_TOP];
     for (int k = 0; k < top; ++k) {
@@ -34,7 +48,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
       for (int e = 0; e < experts; ++e) {
         bool taken = false;
         for (int j = 0; j < k; ++j) taken |= idx[j] == e;
-        if (!taken && (best < 0 || z[e] > bv)) best = e, bv = z[e];
+        if (!taken && (best < 0 || zt[e] > bv)) best = e, bv = zt[e];
       }
       idx[k] = best, val[k] = bv;
     }
@@ -54,10 +68,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
 extern "C" int ns_moe_route(const void* h, int h_stride, const float* wr, const float* br, int* sel, float* wt, int n, int W, int experts,
                             int top, int dtype, hipStream_t stream) {
   if (n <= 0 || W <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > MOE_MAX_TOP || top > experts) return NS_ERR_BAD_ARG;
+  const int blocks = (n + ROUTE_TOK - 1) / ROUTE_TOK;
   if (dtype == NS_DTYPE_F32)
-    moe_route_kernel<float><<<n, 256, 0, stream>>>((const float*)h, h_stride, wr, br, sel, wt, W, experts, top);
+    moe_route_kernel<float><<<blocks, 256, 0, stream>>>((const float*)h, h_stride, wr, br, sel, wt, n, W, experts, top);
   else if (dtype == NS_DTYPE_BF16)
-    moe_route_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)h, h_stride, wr, br, sel, wt, W, experts, top);
+    moe_route_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)h, h_stride, wr, br, sel, wt, n, W, experts, top);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();
@@ -69,59 +84,279 @@ __device__ __forceinline__ float clipped_glu(float g, float u, float limit, floa
   return g / (1.f + expf(-alpha * g)) * (u + 1.f);
 }
 
-// One workgroup a (token, chosen expert): the row in LDS, a wave an inner channel in turn (gate and up together), then a
-// wave an output channel in turn.  out [tokens][top][W] in 32-bit, already times the router's weight.
+// ------------------------------------------------------------------------------------------------ few rows
+// Steps of few rows stream the chosen experts' matrices, each exactly once per (token, expert) that chose it, cut into
+// slices so that the launch fills the chip:
+//   first:  grid (slices of inner channels, top, tokens): the token's row in LDS, a wave an inner channel in turn (its gate row
+//           and its up row together, 16 bytes a lane a load); act [tokens][top][ff] in 32-bit, rounded as a store in the
+//           model's precision would round it
+//   second: grid (slices of output channels, top, tokens): the activations in LDS, a wave an output channel in turn;
+//           out [tokens][top][W] in 32-bit, already times the router's weight
+template <typename T> struct Row8;
+template <> struct Row8<float> {
+  static __device__ __forceinline__ void load(const float* p, float* out) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    out[0] = a.x, out[1] = a.y, out[2] = a.z, out[3] = a.w, out[4] = b.x, out[5] = b.y, out[6] = b.z, out[7] = b.w;
+  }
+};
+template <> struct Row8<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float* out) {
+    typedef bf16_t v8 __attribute__((ext_vector_type(8)));
+    const v8 a = __builtin_nontemporal_load(reinterpret_cast<const v8*>(p));
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[j] = (float)a[j];
+  }
+};
+
+// sum_c w[c] x[c] over a wave; ``vec``: K is a multiple of 8 and the row starts at a multiple of 8 elements of an aligned base
 template <typename T>
-__global__ __launch_bounds__(256) void moe_expert_rows_kernel(const T* __restrict__ h, int h_stride, const T* __restrict__ wg,
-                                                              const T* __restrict__ wu, const T* __restrict__ wd, const int* __restrict__ sel,
-                                                              const float* __restrict__ wt, float* __restrict__ out, int W, int ff, int top,
-                                                              float limit, float alpha) {
-  extern __shared__ float moe_lds[];
-  float* x = moe_lds;      // [W]
-  float* act = x + W;      // [ff]
-  const int t = blockIdx.x, k = blockIdx.y, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE, waves = blockDim.x / NS_WAVE;
+__device__ __forceinline__ float row_dot(const T* __restrict__ w, const float* __restrict__ x, int K, int lane, bool vec) {
+  float acc = 0.f;
+  if (vec) {
+    for (int c = lane * 8; c < K; c += NS_WAVE * 8) {
+      float v[8];
+      Row8<T>::load(w + c, v);
+      const float4 x0 = *reinterpret_cast<const float4*>(x + c), x1 = *reinterpret_cast<const float4*>(x + c + 4);
+      acc = fmaf(v[0], x0.x, acc), acc = fmaf(v[1], x0.y, acc), acc = fmaf(v[2], x0.z, acc), acc = fmaf(v[3], x0.w, acc);
+      acc = fmaf(v[4], x1.x, acc), acc = fmaf(v[5], x1.y, acc), acc = fmaf(v[6], x1.z, acc), acc = fmaf(v[7], x1.w, acc);
+    }
+  } else {
+    for (int c = lane; c < K; c += NS_WAVE) acc = fmaf(to_f(w[c]), x[c], acc);
+  }
+  return wave_sum(acc);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_rows_up_kernel(const T* __restrict__ h, int h_stride, const T* __restrict__ wg, const T* __restrict__ wu,
+                                                          const int* __restrict__ sel, float* __restrict__ act, int W, int ff, int top, int per,
+                                                          float limit, float alpha, int vec) {
+  extern __shared__ __attribute__((aligned(16))) float moe_lds[];  // [W]
+  const int t = blockIdx.z, k = blockIdx.y, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE, waves = blockDim.x / NS_WAVE;
+  const int e = sel[(size_t)t * top + k];
+  for (int c = threadIdx.x; c < W; c += blockDim.x) moe_lds[c] = to_f(h[(size_t)t * h_stride + c]);
+  __syncthreads();
+  const int f0 = blockIdx.x * per, f1 = min(ff, f0 + per);
+  for (int f = f0 + wave; f < f1; f += waves) {
+    const size_t row = ((size_t)e * ff + f) * W;
+    const float g = row_dot(wg + row, moe_lds, W, lane, vec), u = row_dot(wu + row, moe_lds, W, lane, vec);
+    if (lane == 0) act[((size_t)t * top + k) * ff + f] = round_to<T>(clipped_glu(round_to<T>(g), round_to<T>(u), limit, alpha));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_rows_down_kernel(const float* __restrict__ act, const T* __restrict__ wd, const int* __restrict__ sel,
+                                                            const float* __restrict__ wt, float* __restrict__ out, int W, int ff, int top, int per,
+                                                            int vec) {
+  extern __shared__ __attribute__((aligned(16))) float moe_lds[];  // [ff]
+  const int t = blockIdx.z, k = blockIdx.y, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE, waves = blockDim.x / NS_WAVE;
   const int e = sel[(size_t)t * top + k];
   const float share = wt[(size_t)t * top + k];
-  for (int c = threadIdx.x; c < W; c += blockDim.x) x[c] = to_f(h[(size_t)t * h_stride + c]);
+  for (int f = threadIdx.x; f < ff; f += blockDim.x) moe_lds[f] = act[((size_t)t * top + k) * ff + f];
   __syncthreads();
-  const T* g_rows = wg + (size_t)e * ff * W;
-  const T* u_rows = wu + (size_t)e * ff * W;
-  for (int f = wave; f < ff; f += waves) {
-    const T* gr = g_rows + (size_t)f * W;
-    const T* ur = u_rows + (size_t)f * W;
-    float g = 0.f, u = 0.f;
-    for (int c = lane; c < W; c += NS_WAVE) {
-      g = fmaf(to_f(gr[c]), x[c], g);
-      u = fmaf(to_f(ur[c]), x[c], u);
-    }
-    g = wave_sum(g), u = wave_sum(u);
-    if (lane == 0) act[f] = round_to<T>(clipped_glu(round_to<T>(g), round_to<T>(u), limit, alpha));
-  }
-  __syncthreads();
-  const T* d_rows = wd + (size_t)e * W * ff;
-  for (int c = wave; c < W; c += waves) {
-    const T* dr = d_rows + (size_t)c * ff;
-    float y = 0.f;
-    for (int f = lane; f < ff; f += NS_WAVE) y = fmaf(to_f(dr[f]), act[f], y);
-    y = wave_sum(y);
+  const int c0 = blockIdx.x * per, c1 = min(W, c0 + per);
+  for (int c = c0 + wave; c < c1; c += waves) {
+    const float y = row_dot(wd + ((size_t)e * W + c) * ff, moe_lds, ff, lane, vec);
     if (lane == 0) out[((size_t)t * top + k) * W + c] = share * y;
   }
 }
 
+// channels a workgroup takes so that the launch has about 2048 workgroups, a multiple of the four waves
+static int moe_slice(int channels, int rows) {
+  int per = (int)(((long long)channels * rows + 2047) / 2048);
+  per = (per + 3) / 4 * 4;
+  return per < 4 ? 4 : per;
+}
+
 extern "C" int ns_moe_expert_rows(const void* h, int h_stride, const void* wg, const void* wu, const void* wd, const int* sel, const float* wt,
-                                  float* out, int n, int W, int ff, int top, float limit, float alpha, int dtype, hipStream_t stream) {
-  if (n <= 0 || W <= 0 || ff <= 0 || top <= 0 || top > 65535) return NS_ERR_BAD_ARG;
-  const size_t lds = (size_t)(W + ff) * sizeof(float);
-  if (lds > 64 * 1024) return NS_ERR_UNSUPPORTED;
-  dim3 grid(n, top);
-  if (dtype == NS_DTYPE_F32)
-    moe_expert_rows_kernel<float><<<grid, 256, lds, stream>>>((const float*)h, h_stride, (const float*)wg, (const float*)wu, (const float*)wd, sel,
-                                                               wt, out, W, ff, top, limit, alpha);
-  else if (dtype == NS_DTYPE_BF16)
-    moe_expert_rows_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)h, h_stride, (const bf16_t*)wg, (const bf16_t*)wu, (const bf16_t*)wd,
-                                                                sel, wt, out, W, ff, top, limit, alpha);
-  else
+                                  float* act, float* out, int n, int W, int ff, int top, float limit, float alpha, int dtype, hipStream_t stream) {
+  if (n <= 0 || n > 65535 || W <= 0 || ff <= 0 || top <= 0 || top > 65535) return NS_ERR_BAD_ARG;
+  if ((size_t)W * sizeof(float) > 64 * 1024 || (size_t)ff * sizeof(float) > 64 * 1024) return NS_ERR_UNSUPPORTED;
+  const size_t elem = dtype == NS_DTYPE_F32 ? 4 : 2;
+  const int vec_up = W % 8 == 0 && (uintptr_t)wg % (8 * elem) == 0 && (uintptr_t)wu % (8 * elem) == 0;
+  const int vec_down = ff % 8 == 0 && (uintptr_t)wd % (8 * elem) == 0;
+  const int per_f = moe_slice(ff, n * top), per_c = moe_slice(W, n * top);
+  dim3 g1((ff + per_f - 1) / per_f, top, n), g2((W + per_c - 1) / per_c, top, n);
+  if (dtype == NS_DTYPE_F32) {
+    moe_rows_up_kernel<float><<<g1, 256, W * sizeof(float), stream>>>((const float*)h, h_stride, (const float*)wg, (const float*)wu, sel, act, W, ff,
+                                                                       top, per_f, limit, alpha, vec_up);
+    moe_rows_down_kernel<float><<<g2, 256, ff * sizeof(float), stream>>>(act, (const float*)wd, sel, wt, out, W, ff, top, per_c, vec_down);
+  } else if (dtype == NS_DTYPE_BF16) {
+    moe_rows_up_kernel<bf16_t><<<g1, 256, W * sizeof(float), stream>>>((const bf16_t*)h, h_stride, (const bf16_t*)wg, (const bf16_t*)wu, sel, act, W,
+                                                                        ff, top, per_f, limit, alpha, vec_up);
+    moe_rows_down_kernel<bf16_t><<<g2, 256, ff * sizeof(float), stream>>>(act, (const bf16_t*)wd, sel, wt, out, W, ff, top, per_c, vec_down);
+  } else {
     return NS_ERR_UNSUPPORTED;
+  }
+  return ns_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------ many rows
+// Steps of many rows (bfloat16): the (token, chosen expert) pairs are sorted by expert on the device, and every expert's
+// pairs are cut into tiles of 64 rows.  A workgroup takes one tile and 64 output channels and multiplies on the matrix
+// cores (v_mfma_f32_16x16x32_bf16): its four waves own 32 x 32 each, operands come through LDS in pieces of 64 along K,
+// the next piece is fetched into registers while the current one is multiplied.  The host never learns which experts were
+// chosen: the launch has as many tiles as any choice can need (pairs / 64 + experts), and a tile without rows returns.
+//   first:  rows gathered from h by the sorted pairs; gate and up matrices in the same pass; act [pairs sorted][ff] in bfloat16
+//   second: act times the down matrix; out [tokens][top][W] in 32-bit, each row back at its pair and times its weight
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+#define MG_TM 64
+#define MG_TN 64
+#define MG_KC 64
+#define MG_LD (MG_KC + 8)  // bfloat16 values between two rows of a staged tile (padded: neighbouring rows start in other banks)
+
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ sel, int pairs, int experts, int* __restrict__ perm,
+                                                        int* __restrict__ tile_e, int* __restrict__ tile_r0, int* __restrict__ tile_rows,
+                                                        int max_tiles) {
+  __shared__ int cnt[MOE_MAX_EXPERTS], off[MOE_MAX_EXPERTS], cur[MOE_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) cnt[e] = 0, cur[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&cnt[sel[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tiles = 0;
+    for (int e = 0; e < experts; ++e) {
+      off[e] = at;
+      for (int r = 0; r < cnt[e] && tiles < max_tiles; r += MG_TM, ++tiles)
+        tile_e[tiles] = e, tile_r0[tiles] = at + r, tile_rows[tiles] = min(MG_TM, cnt[e] - r);
+      at += cnt[e];
+    }
+    for (; tiles < max_tiles; ++tiles) tile_e[tiles] = -1, tile_r0[tiles] = 0, tile_rows[tiles] = 0;
+  }
+  __syncthreads();
+  // (which pair of an expert gets which of its places depends on timing; a pair's result does not depend on its place)
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = sel[p];
+    perm[off[e] + atomicAdd(&cur[e], 1)] = p;
+  }
+}
+
+template <bool DUAL>
+__global__ __launch_bounds__(256) void moe_group_kernel(const bf16_t* __restrict__ A, int a_stride, const bf16_t* __restrict__ B0,
+                                                        const bf16_t* __restrict__ B1, const int* __restrict__ perm,
+                                                        const int* __restrict__ tile_e, const int* __restrict__ tile_r0,
+                                                        const int* __restrict__ tile_rows, bf16_t* __restrict__ act_out, float* __restrict__ out,
+                                                        const float* __restrict__ wt, int N, int K, int top, float limit, float alpha) {
+  __shared__ __attribute__((aligned(16))) bf16_t As[MG_TM * MG_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Bs[(DUAL ? 2 : 1) * MG_TN * MG_LD];
+  const int tile = blockIdx.y, e = tile_e[tile];
+  if (e < 0) return;
+  const int r0 = tile_r0[tile], rows = tile_rows[tile], n0 = blockIdx.x * MG_TN;
+  const int tid = threadIdx.x, lane = tid % NS_WAVE, wave = tid / NS_WAVE, r = lane % 16, g = lane / 16;
+  const int wm = wave / 2, wn = wave % 2;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  // the two pieces (8 values along K) of each staged tile that this thread fetches: rows tid / 8 and tid / 8 + 32, piece tid % 8
+  const int kp = (tid % 8) * 8;
+  const bf16_t* arow[2];
+  const bf16_t* brow0[2];
+  const bf16_t* brow1[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = tid / 8 + 32 * i;
+    const int slot = r0 + row;
+    arow[i] = row < rows ? A + (size_t)(DUAL ? perm[slot] / top : slot) * a_stride : nullptr;
+    const int col = n0 + row;
+    brow0[i] = col < N ? B0 + ((size_t)e * N + col) * K : nullptr;
+    brow1[i] = (DUAL && col < N) ? B1 + ((size_t)e * N + col) * K : nullptr;
+  }
+  bf16x8 pa[2], pb0[2], pb1[2];
+  auto fetch = [&](int k0) {
+    const bool ok = k0 + kp < K;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      pa[i] = (ok && arow[i]) ? *reinterpret_cast<const bf16x8*>(arow[i] + k0 + kp) : zero;
+      pb0[i] = (ok && brow0[i]) ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(brow0[i] + k0 + kp)) : zero;
+      if (DUAL) pb1[i] = (ok && brow1[i]) ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(brow1[i] + k0 + kp)) : zero;
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int at = (tid / 8 + 32 * i) * MG_LD + kp;
+      *reinterpret_cast<bf16x8*>(As + at) = pa[i];
+      *reinterpret_cast<bf16x8*>(Bs + at) = pb0[i];
+      if (DUAL) *reinterpret_cast<bf16x8*>(Bs + MG_TN * MG_LD + at) = pb1[i];
+    }
+  };
+
+  f32x4 acc0[2][2], acc1[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc0[i][j] = f32x4{0.f, 0.f, 0.f, 0.f}, acc1[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += MG_KC) {
+    stage();
+    __syncthreads();
+    if (k0 + MG_KC < K) fetch(k0 + MG_KC);
+#pragma unroll
+    for (int ks = 0; ks < MG_KC; ks += 32) {
+      bf16x8 af[2], bf0[2], bf1[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        af[i] = *reinterpret_cast<const bf16x8*>(As + (32 * wm + 16 * i + r) * MG_LD + ks + 8 * g);
+        bf0[i] = *reinterpret_cast<const bf16x8*>(Bs + (32 * wn + 16 * i + r) * MG_LD + ks + 8 * g);
+        if (DUAL) bf1[i] = *reinterpret_cast<const bf16x8*>(Bs + MG_TN * MG_LD + (32 * wn + 16 * i + r) * MG_LD + ks + 8 * g);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          acc0[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf0[j], acc0[i][j], 0, 0, 0);
+          if (DUAL) acc1[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf1[j], acc1[i][j], 0, 0, 0);
+        }
+    }
+    __syncthreads();
+  }
+  // element q of a lane's sums is row 4 g + q of the 16 x 16 block, column r
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int row = 32 * wm + 16 * i + 4 * g + q;
+      if (row >= rows) continue;
+      const int slot = r0 + row;
+      const int pair = DUAL ? 0 : perm[slot];
+      const float share = DUAL ? 0.f : wt[pair];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int col = n0 + 32 * wn + 16 * j + r;
+        if (col >= N) continue;
+        if (DUAL)
+          act_out[(size_t)slot * N + col] = from_f<bf16_t>(clipped_glu(round_to<bf16_t>(acc0[i][j][q]), round_to<bf16_t>(acc1[i][j][q]), limit, alpha));
+        else
+          out[(size_t)pair * N + col] = share * acc0[i][j][q];
+      }
+    }
+}
+
+// tiles that any choice of experts can need
+extern "C" int ns_moe_group_tiles(int pairs, int experts) { return (pairs + MG_TM - 1) / MG_TM + experts; }
+
+// ``ints``: scratch of pairs + 3 * ns_moe_group_tiles(pairs, experts) 32-bit words; ``act``: bfloat16 [pairs][ff]
+extern "C" int ns_moe_expert_groups(const void* h, int h_stride, const void* wg, const void* wu, const void* wd, const int* sel, const float* wt,
+                                    int* ints, void* act, float* out, int n, int W, int ff, int top, int experts, float limit, float alpha,
+                                    hipStream_t stream) {
+  if (n <= 0 || W <= 0 || ff <= 0 || top <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS) return NS_ERR_BAD_ARG;
+  if (W % 8 || ff % 8 || h_stride % 8 || (uintptr_t)h % 16 || (uintptr_t)wg % 16 || (uintptr_t)wu % 16 || (uintptr_t)wd % 16 || (uintptr_t)act % 16)
+    return NS_ERR_UNSUPPORTED;
+  const long long pairs = (long long)n * top;
+  if (pairs > (1 << 24)) return NS_ERR_UNSUPPORTED;
+  const int tiles = ns_moe_group_tiles((int)pairs, experts);
+  if (tiles > 65535) return NS_ERR_UNSUPPORTED;
+  int* perm = ints;
+  int* tile_e = ints + pairs;
+  int* tile_r0 = tile_e + tiles;
+  int* tile_rows = tile_r0 + tiles;
+  moe_sort_kernel<<<1, 1024, 0, stream>>>(sel, (int)pairs, experts, perm, tile_e, tile_r0, tile_rows, tiles);
+  dim3 g1((ff + MG_TN - 1) / MG_TN, tiles), g2((W + MG_TN - 1) / MG_TN, tiles);
+  moe_group_kernel<true><<<g1, 256, 0, stream>>>((const bf16_t*)h, h_stride, (const bf16_t*)wg, (const bf16_t*)wu, perm, tile_e, tile_r0, tile_rows,
+                                                  (bf16_t*)act, nullptr, nullptr, ff, W, top, limit, alpha);
+  moe_group_kernel<false><<<g2, 256, 0, stream>>>((const bf16_t*)act, ff, (const bf16_t*)wd, nullptr, perm, tile_e, tile_r0, tile_rows, nullptr, out,
+                                                   wt, W, ff, top, limit, alpha);
   return ns_launch_status();
 }
 
@@ -201,44 +436,28 @@ extern "C" int ns_scaled_sum(void* out, const void* a, const void* b, const void
 }
 
 // The per-layer token input: y = W_proj (gelu_tanh(W_gate x) * e) with e = table[token] (this layer's ``dim`` columns of a
-// row).  One workgroup a token: a wave a gate channel in turn, then a thread an output channel.
+// row).  The two products are the framework's; between them: out[t][j] = gelu_tanh(g[t][j]) * table[ids[t]][j].
 template <typename T>
-__global__ __launch_bounds__(256) void token_side_kernel(T* __restrict__ out, const T* __restrict__ x, int x_stride, const int* __restrict__ ids,
-                                                         const T* __restrict__ table, const T* __restrict__ wg, const T* __restrict__ wp, int W,
-                                                         int dim) {
-  extern __shared__ float side_lds[];  // [dim]
-  const int t = blockIdx.x, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE, waves = blockDim.x / NS_WAVE;
-  const T* xr = x + (size_t)t * x_stride;
-  const T* e = table + (size_t)ids[t] * dim;
-  for (int j = wave; j < dim; j += waves) {
-    const T* w = wg + (size_t)j * W;
-    float acc = 0.f;
-    for (int c = lane; c < W; c += NS_WAVE) acc = fmaf(to_f(w[c]), to_f(xr[c]), acc);
-    acc = round_to<T>(wave_sum(acc));
-    if (lane == 0) {
-      const float gl = 0.5f * acc * (1.f + tanhf(0.7978845608028654f * (acc + 0.044715f * acc * acc * acc)));
-      side_lds[j] = round_to<T>(round_to<T>(gl) * to_f(e[j]));
-    }
-  }
-  __syncthreads();
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    const T* w = wp + (size_t)c * dim;
-    float acc = 0.f;
-    for (int j = 0; j < dim; ++j) acc = fmaf(to_f(w[j]), side_lds[j], acc);
-    out[(size_t)t * W + c] = from_f<T>(acc);
+__global__ void gelu_gather_mul_kernel(T* __restrict__ out, const T* __restrict__ g, int g_stride, const int* __restrict__ ids,
+                                       const T* __restrict__ table, int dim, size_t count) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = i / dim, j = i % dim;
+    const float z = to_f(g[t * g_stride + j]);
+    const float gl = 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    out[i] = from_f<T>(round_to<T>(gl) * to_f(table[(size_t)ids[t] * dim + j]));
   }
 }
 
-extern "C" int ns_token_side(void* out, const void* x, int x_stride, const int* ids, const void* table, const void* wg, const void* wp, int n,
-                             int W, int dim, int dtype, hipStream_t stream) {
-  if (n <= 0 || W <= 0 || dim <= 0 || dim > 8192) return NS_ERR_BAD_ARG;
-  const size_t lds = (size_t)dim * sizeof(float);
+extern "C" int ns_gelu_gather_mul(void* out, const void* g, int g_stride, const int* ids, const void* table, int n, int dim, int dtype,
+                                  hipStream_t stream) {
+  if (n <= 0 || dim <= 0) return NS_ERR_BAD_ARG;
+  const size_t count = (size_t)n * dim;
+  size_t blocks = (count + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
   if (dtype == NS_DTYPE_F32)
-    token_side_kernel<float><<<n, 256, lds, stream>>>((float*)out, (const float*)x, x_stride, ids, (const float*)table, (const float*)wg,
-                                                       (const float*)wp, W, dim);
+    gelu_gather_mul_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)out, (const float*)g, g_stride, ids, (const float*)table, dim, count);
   else if (dtype == NS_DTYPE_BF16)
-    token_side_kernel<bf16_t><<<n, 256, lds, stream>>>((bf16_t*)out, (const bf16_t*)x, x_stride, ids, (const bf16_t*)table, (const bf16_t*)wg,
-                                                        (const bf16_t*)wp, W, dim);
+    gelu_gather_mul_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)g, g_stride, ids, (const bf16_t*)table, dim, count);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();

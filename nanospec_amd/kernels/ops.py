@@ -1140,30 +1140,65 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, 
 
 
 def moe_expert_rows(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
-                    limit: float, alpha: float, out: torch.Tensor) -> torch.Tensor:
-    """out[t, k] = weights[t, k] * expert sel[t, k] of h[t]: one workgroup per (token, chosen expert).  ``gate``, ``up``
-    [experts, ff, W], ``down`` [experts, W, ff] in the dtype of ``h``; ``out`` float32 [tokens, top, W]."""
-    _gpu(h, gate, up, down, sel, weights, out)
-    _f32(out, "out"), _f32(weights, "weights"), _i32(sel, "sel")
+                    limit: float, alpha: float, act: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, k] = weights[t, k] * expert sel[t, k] of h[t], for few rows: every (token, chosen expert) streams that expert's
+    matrices, cut into slices over many workgroups.  ``gate``, ``up`` [experts, ff, W], ``down`` [experts, W, ff] in the dtype
+    of ``h``; ``act`` float32 [tokens, top, ff] (scratch); ``out`` float32 [tokens, top, W]."""
+    _gpu(h, gate, up, down, sel, weights, act, out)
+    _f32(out, "out"), _f32(act, "act"), _f32(weights, "weights"), _i32(sel, "sel")
     n, W = h.shape
     experts, ff = gate.shape[0], gate.shape[1]
     top = sel.shape[1]
     if (h.stride(1) != 1 or gate.shape != (experts, ff, W) or up.shape != gate.shape or down.shape != (experts, W, ff) or sel.shape != (n, top)
-            or weights.shape != (n, top) or out.shape != (n, top, W) or any(t.dtype != h.dtype or not t.is_contiguous() for t in (gate, up, down))):
-        raise KernelRefused("moe_expert_rows: gate and up [experts, ff, W], down [experts, W, ff] in the dtype of h; out float32 [tokens, top, W]")
-    _check(build.core().ns_moe_expert_rows(_ptr(h), c_int(h.stride(0)), _ptr(gate), _ptr(up), _ptr(down), _ptr(sel), _ptr(weights), _ptr(out),
-                                           c_int(n), c_int(W), c_int(ff), c_int(top), c_float(limit), c_float(alpha), c_int(_dtype_code(h)),
-                                           _stream()), "moe_expert_rows")
+            or weights.shape != (n, top) or out.shape != (n, top, W) or act.shape != (n, top, ff)
+            or any(t.dtype != h.dtype or not t.is_contiguous() for t in (gate, up, down))):
+        raise KernelRefused("moe_expert_rows: gate and up [experts, ff, W], down [experts, W, ff] in the dtype of h; act [tokens, top, ff] and out [tokens, top, W] float32")
+    _check(build.core().ns_moe_expert_rows(_ptr(h), c_int(h.stride(0)), _ptr(gate), _ptr(up), _ptr(down), _ptr(sel), _ptr(weights), _ptr(act),
+                                           _ptr(out), c_int(n), c_int(W), c_int(ff), c_int(top), c_float(limit), c_float(alpha),
+                                           c_int(_dtype_code(h)), _stream()), "moe_expert_rows")
+    return out
+
+
+def moe_groups_take(h: torch.Tensor, ff: int) -> bool:
+    """Whether the matrix-core kernels for many rows take this input: bfloat16, sizes in multiples of 8."""
+    return h.dtype == torch.bfloat16 and h.shape[1] % 8 == 0 and ff % 8 == 0 and h.stride(0) % 8 == 0 and h.data_ptr() % 16 == 0
+
+
+def moe_expert_groups(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
+                      limit: float, alpha: float, ints: torch.Tensor, act: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """The same result for many rows in bfloat16: the pairs are sorted by expert on the device and every expert multiplies
+    its rows in tiles on the matrix cores.  ``ints`` int32 [tokens * top + 3 * moe_group_tiles] and ``act`` bfloat16
+    [tokens * top, ff] are scratch."""
+    _gpu(h, gate, up, down, sel, weights, ints, act, out)
+    _f32(out, "out"), _f32(weights, "weights"), _i32(sel, "sel"), _i32(ints, "ints")
+    n, W = h.shape
+    experts, ff = gate.shape[0], gate.shape[1]
+    top = sel.shape[1]
+    tiles = int(build.core().ns_moe_group_tiles(c_int(n * top), c_int(experts)))
+    if (not moe_groups_take(h, ff) or h.stride(1) != 1 or gate.shape != (experts, ff, W) or up.shape != gate.shape or down.shape != (experts, W, ff)
+            or sel.shape != (n, top) or weights.shape != (n, top) or out.shape != (n, top, W) or act.shape != (n * top, ff) or act.dtype != h.dtype
+            or not act.is_contiguous() or ints.numel() < n * top + 3 * tiles or any(t.dtype != h.dtype or not t.is_contiguous() for t in (gate, up, down))):
+        raise KernelRefused("moe_expert_groups: bfloat16 operands with sizes in multiples of 8, act [pairs, ff], ints [pairs + 3 tiles]")
+    _check(build.core().ns_moe_expert_groups(_ptr(h), c_int(h.stride(0)), _ptr(gate), _ptr(up), _ptr(down), _ptr(sel), _ptr(weights), _ptr(ints),
+                                             _ptr(act), _ptr(out), c_int(n), c_int(W), c_int(ff), c_int(top), c_int(experts), c_float(limit),
+                                             c_float(alpha), _stream()), "moe_expert_groups")
     return out
 
 
 def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
                 limit: float, alpha: float, take) -> torch.Tensor:
-    """The chosen experts' weighted outputs, float32 [tokens, top, W], by the kernel that suits the number of rows.
-    ``take(shape, dtype)`` gives scratch that lives as long as the result."""
+    """The chosen experts' weighted outputs, float32 [tokens, top, W], by the kernels that suit the number of rows: with
+    fewer (token, expert) pairs than experts every pair streams its expert's matrices; from there on the sorted, tiled
+    product reads every matrix at most once.  ``take(shape, dtype)`` gives scratch that lives as long as the result."""
     n, W = h.shape
+    experts, ff = gate.shape[0], gate.shape[1]
     top = sel.shape[1]
-    return moe_expert_rows(h, gate, up, down, sel, weights, limit, alpha, take((n, top, W), torch.float32))
+    out = take((n, top, W), torch.float32)
+    if n * top >= max(experts, 16) and moe_groups_take(h, ff):
+        tiles = int(build.core().ns_moe_group_tiles(c_int(n * top), c_int(experts)))
+        return moe_expert_groups(h, gate, up, down, sel, weights, limit, alpha, take((n * top + 3 * tiles,), torch.int32),
+                                 take((n * top, ff), h.dtype), out)
+    return moe_expert_rows(h, gate, up, down, sel, weights, limit, alpha, take((n, top, ff), torch.float32), out)
 
 
 def clipped_glu(gu: torch.Tensor, limit: float, alpha: float, out: torch.Tensor) -> torch.Tensor:
@@ -1204,17 +1239,16 @@ def scaled_sum(a: torch.Tensor, b: torch.Tensor, sa: float, sb: float, out: torc
     return out
 
 
-def token_side(x: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, gate: torch.Tensor, proj: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t] = proj (gelu_tanh(gate x[t]) * table[ids[t]]): ``table`` [vocab, dim], ``gate`` [dim, W], ``proj`` [W, dim]."""
-    _gpu(x, ids, table, gate, proj, out)
+def gelu_gather_mul(g: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = gelu_tanh(g[t]) * table[ids[t]]: ``g`` [tokens, dim] (may be a column slice), ``table`` [vocab, dim]."""
+    _gpu(g, ids, table, out)
     _i32(ids, "ids")
-    n, W = x.shape
-    dim = table.shape[1]
-    if (x.stride(1) != 1 or ids.numel() != n or gate.shape != (dim, W) or proj.shape != (W, dim) or out.shape != (n, W) or not out.is_contiguous()
-            or any(t.dtype != x.dtype or not t.is_contiguous() for t in (table, gate, proj)) or out.dtype != x.dtype):
-        raise KernelRefused("token_side: table [vocab, dim], gate [dim, W], proj [W, dim], all in the dtype of x")
-    _check(build.core().ns_token_side(_ptr(out), _ptr(x), c_int(x.stride(0)), _ptr(ids), _ptr(table), _ptr(gate), _ptr(proj), c_int(n), c_int(W),
-                                      c_int(dim), c_int(_dtype_code(x)), _stream()), "token_side")
+    n, dim = out.shape
+    if (g.shape != (n, dim) or g.stride(1) != 1 or ids.numel() != n or table.dim() != 2 or table.shape[1] != dim or not table.is_contiguous()
+            or not out.is_contiguous() or table.dtype != g.dtype or out.dtype != g.dtype):
+        raise KernelRefused("gelu_gather_mul: g and out [tokens, dim], table [vocab, dim], all of one dtype")
+    _check(build.core().ns_gelu_gather_mul(_ptr(out), _ptr(g), c_int(g.stride(0)), _ptr(ids), _ptr(table), c_int(n), c_int(dim),
+                                           c_int(_dtype_code(g)), _stream()), "gelu_gather_mul")
     return out
 
 

@@ -522,8 +522,8 @@ def test_the_running_maximum_starts_at_zero():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("W,n,top,ff,limit,shared", [(90, 5, 2, 40, 1.2, (56, 2.0)), (64, 1, 1, 48, 3.0, None), (128, 16, 3, 32, 1.5, (64, 7.0)),
-                                                      (50, 7, 7, 24, 0.5, None), (256, 64, 4, 128, 1.5, (256, 1.5))])
-@pytest.mark.parametrize("rows", [1, 7, 300])
+                                                      (50, 7, 7, 24, 0.5, None), (256, 64, 4, 128, 1.5, (256, 1.5)), (200, 3, 2, 72, 1.0, None), (1024, 8, 2, 328, 2.0, None)])
+@pytest.mark.parametrize("rows", [1, 7, 300, 1000])
 def test_mixture_of_experts_through_the_part(dtype, W, n, top, ff, limit, shared, rows):
     from nanospec_amd.config.spec import ClippedGLUSpec, MoESpec
     from nanospec_amd.engine.arena import Arena
@@ -576,17 +576,30 @@ def test_router_weights_are_the_softmax_over_the_chosen():
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("W,dim,vocab", [(90, 6, 50), (64, 1, 9), (128, 32, 200), (50, 100, 30)])
 def test_token_input_of_a_layer(dtype, W, dim, vocab):
-    from nanospec_amd.kernels import ops
+    """The part as the framework builds it (two products and the kernel between them), its columns in the middle of a
+    table that other layers share."""
+    from nanospec_amd.config.spec import TokenSideSpec
+    from nanospec_amd.engine.arena import Arena
+    from nanospec_amd.parts import registry
 
     g = torch.Generator().manual_seed(W + dim)
-    table, gate, proj = (3 * torch.randn(vocab, dim, generator=g)).to(dtype), (0.3 * torch.randn(dim, W, generator=g)).to(dtype), torch.randn(W, dim, generator=g).to(dtype)
-    x = torch.randn(11, W, generator=g).to(dtype)
-    ids = torch.randint(0, vocab, (11,), generator=g)
-    ref = (pp.gelu_tanh(x.double() @ gate.double().T) * table.double()[ids]) @ proj.double().T
-    out = torch.empty(11, W, dtype=dtype, device=DEV)
-    ops.token_side(x.to(DEV), ids.to(DEV, torch.int32), table.to(DEV), gate.to(DEV), proj.to(DEV), out)
-    scale = ref.abs().max()
-    assert (out.cpu().double() - ref).abs().max() <= (2e-5 if dtype == torch.float32 else 3e-2) * scale
+    whole = (3 * torch.randn(vocab, 3 * dim, generator=g)).to(dtype)
+    gate, proj = (0.3 * torch.randn(dim, W, generator=g)).to(dtype), torch.randn(W, dim, generator=g).to(dtype)
+    part = registry.build("ffn", TokenSideSpec(hidden=W, vocab=vocab, dim=dim, offset=dim, table_dim=3 * dim), "s.")
+    tensors = {"side.embed": whole, "s.gate": gate, "s.proj": proj}
+    part.load(lambda name: tensors[name], dtype, DEV)
+    for n in (1, 11, 200):
+        x = torch.randn(n, W, generator=g).to(dtype)
+        ids = torch.randint(0, vocab, (n,), generator=g)
+        ref = (pp.gelu_tanh(x.double() @ gate.double().T) * whole.double()[ids][:, dim : 2 * dim]) @ proj.double().T
+
+        class Ctx:
+            captured = False
+
+        ctx = Ctx()
+        ctx.arena, ctx.token_ids = Arena(torch.device(DEV)), ids.to(DEV, torch.int32)
+        out = part.forward(ctx, x.to(DEV))
+        assert (out.cpu().double() - ref).abs().max() <= (2e-5 if dtype == torch.float32 else 3e-2) * ref.abs().max()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
