@@ -9,72 +9,92 @@
 #define MOE_MAX_EXPERTS 1024
 #define MOE_MAX_TOP 32
 
-// One workgroup takes ROUTE_TOK tokens: every wave takes experts in turn and reads an expert's row once for all of the
-// tokens; one thread a token then chooses.
+// Two kernels.  Logits: a workgroup takes ROUTE_TOK tokens and four experts, a wave an expert: it reads the expert's row
+// once (16 bytes a lane a load where the sizes allow) for all of its tokens.  Choice: a thread a token.
 #define ROUTE_TOK 8
 template <typename T>
-__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, int h_stride, const float* __restrict__ wr,
-                                                        const float* __restrict__ br, int* __restrict__ sel, float* __restrict__ wt,
-                                                        int n, int W, int experts, int top) {
-  __shared__ float z[ROUTE_TOK][MOE_MAX_EXPERTS];
-  const int t0 = blockIdx.x * ROUTE_TOK, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE, waves = blockDim.x / NS_WAVE;
+__global__ __launch_bounds__(256) void moe_logits_kernel(const T* __restrict__ h, int h_stride, const float* __restrict__ wr,
+                                                         const float* __restrict__ br, float* __restrict__ z, int n, int W, int experts, int vec) {
+  const int t0 = blockIdx.x * ROUTE_TOK, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE;
+  const int e = blockIdx.y * (blockDim.x / NS_WAVE) + wave;
+  if (e >= experts) return;
   const int nt = min(ROUTE_TOK, n - t0);
-  for (int e = wave; e < experts; e += waves) {
-    const float* w = wr + (size_t)e * W;
-    float acc[ROUTE_TOK];
+  const float* w = wr + (size_t)e * W;
+  float acc[ROUTE_TOK];
 #pragma unroll
-    for (int i = 0; i < ROUTE_TOK; ++i) acc[i] = 0.f;
+  for (int i = 0; i < ROUTE_TOK; ++i) acc[i] = 0.f;
+  if (vec) {
+#pragma unroll 2
+    for (int c = lane * 4; c < W; c += NS_WAVE * 4) {
+      const float4 wc = *reinterpret_cast<const float4*>(w + c);
+#pragma unroll
+      for (int i = 0; i < ROUTE_TOK; ++i)
+        if (i < nt) {
+          const T* x = h + (size_t)(t0 + i) * h_stride + c;
+          acc[i] = fmaf(to_f(x[0]), wc.x, acc[i]), acc[i] = fmaf(to_f(x[1]), wc.y, acc[i]);
+          acc[i] = fmaf(to_f(x[2]), wc.z, acc[i]), acc[i] = fmaf(to_f(x[3]), wc.w, acc[i]);
+        }
+    }
+  } else {
     for (int c = lane; c < W; c += NS_WAVE) {
       const float wc = w[c];
 #pragma unroll
       for (int i = 0; i < ROUTE_TOK; ++i)
         if (i < nt) acc[i] = fmaf(to_f(h[(size_t)(t0 + i) * h_stride + c]), wc, acc[i]);
     }
-#pragma unroll
-    for (int i = 0; i < ROUTE_TOK; ++i) {
-      const float v = wave_sum(acc[i]);
-      if (lane == 0) z[i][e] = v + (br ? br[e] : 0.f);
-    }
   }
-  __syncthreads();
-  if (threadIdx.x < nt) {
-    const int t = t0 + threadIdx.x;
-    const float* zt = z[threadIdx.x];
-    int idx[MOE_MAX_TOP];
-    float val[MOE_MAX_TOP];
-    for (int k = 0; k < top; ++k) {
-      int best = -1;
-      float bv = -INFINITY;
-      for (int e = 0; e < experts; ++e) {
-        bool taken = false;
-        for (int j = 0; j < k; ++j) taken |= idx[j] == e;
-        if (!taken && (best < 0 || zt[e] > bv)) best = e, bv = zt[e];
-      }
-      idx[k] = best, val[k] = bv;
-    }
-    float sum = 0.f;
-    const float largest = val[0];
-    for (int k = 0; k < top; ++k) {
-      val[k] = expf(val[k] - largest);
-      sum += val[k];
-    }
-    for (int k = 0; k < top; ++k) {
-      sel[(size_t)t * top + k] = idx[k];
-      wt[(size_t)t * top + k] = val[k] / sum;
-    }
+#pragma unroll
+  for (int i = 0; i < ROUTE_TOK; ++i) {
+    const float v = wave_sum(acc[i]);
+    if (lane == 0 && i < nt) z[(size_t)(t0 + i) * experts + e] = v + (br ? br[e] : 0.f);
   }
 }
 
-extern "C" int ns_moe_route(const void* h, int h_stride, const float* wr, const float* br, int* sel, float* wt, int n, int W, int experts,
+__global__ __launch_bounds__(64) void moe_choose_kernel(const float* __restrict__ z, int* __restrict__ sel, float* __restrict__ wt, int n,
+                                                        int experts, int top) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const float* zt = z + (size_t)t * experts;
+  int idx[MOE_MAX_TOP];
+  float val[MOE_MAX_TOP];
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < experts; ++e) {
+      bool taken = false;
+      for (int j = 0; j < k; ++j) taken |= idx[j] == e;
+      const float v = zt[e];
+      if (!taken && (best < 0 || v > bv)) best = e, bv = v;
+    }
+    idx[k] = best, val[k] = bv;
+  }
+  float sum = 0.f;
+  const float largest = val[0];
+  for (int k = 0; k < top; ++k) {
+    val[k] = expf(val[k] - largest);
+    sum += val[k];
+  }
+  for (int k = 0; k < top; ++k) {
+    sel[(size_t)t * top + k] = idx[k];
+    wt[(size_t)t * top + k] = val[k] / sum;
+  }
+}
+
+// ``z``: scratch, float32 [n][experts]
+extern "C" int ns_moe_route(const void* h, int h_stride, const float* wr, const float* br, float* z, int* sel, float* wt, int n, int W, int experts,
                             int top, int dtype, hipStream_t stream) {
   if (n <= 0 || W <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > MOE_MAX_TOP || top > experts) return NS_ERR_BAD_ARG;
-  const int blocks = (n + ROUTE_TOK - 1) / ROUTE_TOK;
+  dim3 grid((n + ROUTE_TOK - 1) / ROUTE_TOK, (experts + 3) / 4);
+  if (grid.y > 65535) return NS_ERR_UNSUPPORTED;
+  const size_t elem = dtype == NS_DTYPE_F32 ? 4 : 2;
+  const int vec = W % 4 == 0 && h_stride % 4 == 0 && (uintptr_t)wr % 16 == 0 && (uintptr_t)h % (4 * elem) == 0;
   if (dtype == NS_DTYPE_F32)
-    moe_route_kernel<float><<<blocks, 256, 0, stream>>>((const float*)h, h_stride, wr, br, sel, wt, n, W, experts, top);
+    moe_logits_kernel<float><<<grid, 256, 0, stream>>>((const float*)h, h_stride, wr, br, z, n, W, experts, vec);
   else if (dtype == NS_DTYPE_BF16)
-    moe_route_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)h, h_stride, wr, br, sel, wt, n, W, experts, top);
+    moe_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)h, h_stride, wr, br, z, n, W, experts, vec);
   else
     return NS_ERR_UNSUPPORTED;
+  moe_choose_kernel<<<(n + 63) / 64, 64, 0, stream>>>(z, sel, wt, n, experts, top);
   return ns_launch_status();
 }
 

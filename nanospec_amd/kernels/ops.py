@@ -1126,16 +1126,21 @@ def memory_scan(proj: torch.Tensor, offsets: tuple[int, int, int, int, int], gat
 # ------------------------------------------------------------------------------------------------ mixture of experts
 
 
-def moe_route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, top: int, sel: torch.Tensor, weights: torch.Tensor) -> None:
+def moe_route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, top: int, sel: torch.Tensor, weights: torch.Tensor,
+              logits: torch.Tensor | None = None) -> None:
     """Router logits z = router h + bias in 32-bit (``router`` float32 [experts, W]); ``sel`` int32 [tokens, top] receives the
-    experts with the largest logits in falling order, ``weights`` float32 [tokens, top] the soft-max over those logits."""
-    _gpu(h, router, bias, sel, weights)
+    experts with the largest logits in falling order, ``weights`` float32 [tokens, top] the soft-max over those logits.
+    ``logits``: float32 [tokens, experts], receives z (scratch if the caller has no use for it)."""
+    _gpu(h, router, bias, sel, weights, logits)
     _f32(router, "router"), _f32(weights, "weights"), _i32(sel, "sel")
     n, W = h.shape
     experts = router.shape[0]
-    if h.stride(1) != 1 or router.shape != (experts, W) or sel.shape != (n, top) or weights.shape != (n, top) or (bias is not None and _f32(bias, "bias").numel() != experts):
-        raise KernelRefused("moe_route: h [tokens, W], router [experts, W], bias [experts], sel and weights [tokens, top]")
-    _check(build.core().ns_moe_route(_ptr(h), c_int(h.stride(0)), _ptr(router), _ptr(bias), _ptr(sel), _ptr(weights), c_int(n), c_int(W),
+    if logits is None:
+        logits = torch.empty((n, experts), dtype=torch.float32, device=h.device)
+    if (h.stride(1) != 1 or router.shape != (experts, W) or not router.is_contiguous() or sel.shape != (n, top) or weights.shape != (n, top)
+            or (bias is not None and _f32(bias, "bias").numel() != experts) or _f32(logits, "logits").shape != (n, experts) or not logits.is_contiguous()):
+        raise KernelRefused("moe_route: h [tokens, W], router [experts, W], bias [experts], sel and weights [tokens, top], logits [tokens, experts]")
+    _check(build.core().ns_moe_route(_ptr(h), c_int(h.stride(0)), _ptr(router), _ptr(bias), _ptr(logits), _ptr(sel), _ptr(weights), c_int(n), c_int(W),
                                      c_int(experts), c_int(top), c_int(_dtype_code(h)), _stream()), "moe_route")
 
 

@@ -67,7 +67,7 @@ class MoE:
         s = self.spec
         n, take = x.shape[0], ctx.arena.take
         sel, wt = take((n, s.top), torch.int32), take((n, s.top), torch.float32)
-        ops.moe_route(x, self.router, self.router_bias, s.top, sel, wt)
+        ops.moe_route(x, self.router, self.router_bias, s.top, sel, wt, logits=take((n, s.experts), torch.float32))
         base = None
         if s.shared is not None:
             sf = s.shared.intermediate
