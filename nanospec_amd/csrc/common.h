@@ -31,6 +31,24 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// The sum of a value over RGC neighbouring lanes (a power of two; the group starts at a multiple of RGC), in all of them.  Up to 16 lanes lie in one row of the
+// wave, where a lane reads its partner through the data path of the vector unit itself (quad permutations, then the
+// mirrored half row and row: any partner in the other half will do for a sum); wider groups go on through LDS's crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_read(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int RGC>
+__device__ __forceinline__ float group_sum(float v) {
+  if constexpr (RGC >= 2) v += dpp_read<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+  if constexpr (RGC >= 4) v += dpp_read<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  if constexpr (RGC >= 8) v += dpp_read<0x141>(v);  // row_half_mirror
+  if constexpr (RGC >= 16) v += dpp_read<0x140>(v); // row_mirror
+#pragma unroll
+  for (int o = 16; o < RGC; o <<= 1) v += __shfl_xor(v, o, NS_WAVE);
+  return v;
+}
+
 // Block-wide reductions for blocks of up to 1024 threads; `scratch` holds >= 16 floats of LDS.
 // Every thread gets the result.  The order of the additions is fixed by the thread layout only.
 __device__ __forceinline__ float block_sum(float v, float* scratch) {

@@ -199,24 +199,6 @@ extern "C" int ns_delta_prep(float* qkv, int C, float* g, float* beta, const voi
 // current stage's tokens are worked through from LDS, and then written to the other LDS buffer.  The arithmetic of a
 // token is the same whatever the stage it falls into: results do not depend on how a prompt was cut.
 // ------------------------------------------------------------------------------------------------
-// The sum of a value over the RG neighbouring lanes of a column, in all of them.  Up to 16 lanes lie in one row of the
-// wave, where a lane reads its partner through the data path of the vector unit itself (quad permutations, then the
-// mirrored half row and row: any partner in the other half will do for a sum); wider groups go on through LDS's crossbar.
-template <int CTRL>
-__device__ __forceinline__ float dpp_read(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
-template <int RGC>
-__device__ __forceinline__ float group_sum(float v) {
-  if constexpr (RGC >= 2) v += dpp_read<0xB1>(v);   // quad_perm [1, 0, 3, 2]
-  if constexpr (RGC >= 4) v += dpp_read<0x4E>(v);   // quad_perm [2, 3, 0, 1]
-  if constexpr (RGC >= 8) v += dpp_read<0x141>(v);  // row_half_mirror
-  if constexpr (RGC >= 16) v += dpp_read<0x140>(v); // row_mirror
-#pragma unroll
-  for (int o = 16; o < RGC; o <<= 1) v += __shfl_xor(v, o, NS_WAVE);
-  return v;
-}
-
 #define ND_PITCH (ND_ROWS + 4)                     // floats between two row groups' channels in LDS
 #define ND_STAGE_FLOATS 6144                       // floats of one stage in LDS (two stages are held)
 #define ND_STAGE_REGS (ND_STAGE_FLOATS / 1024)     // of which each of the 256 threads fetches this many groups of four

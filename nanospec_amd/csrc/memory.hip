@@ -8,7 +8,7 @@
 // result of one stacked product), in the model's precision; everything from there on is 32-bit.
 //
 // A column of S never meets another column, so a wave owns 64 / TPC columns and the TPC lanes of a column hold 8 key
-// channels each; their partial sums meet by lane exchange.  Every column's lanes also carry n (the same in all columns),
+// channels each; their partial sums meet through the vector unit's lane permutations (``group_sum``).  Every column's lanes also carry n (the same in all columns),
 // so no wave waits for another.  A workgroup is four waves that share the staged operands: the next block of tokens is
 // fetched into registers while the current block is worked through from LDS.
 //
@@ -151,34 +151,53 @@ __global__ __launch_bounds__(MM_THREADS) void memory_scan_kernel(const MemoryPar
   fetch(t0);
   stage();
   __syncthreads();
+  constexpr int UN = 4;  // tokens worked through together: only m, S and n pass from token to token, the rest overlaps
+  static_assert(TB % UN == 0, "a block of tokens is whole groups");
   for (int t = t0; t < t1; t += TB) {
     if (t + TB < t1) fetch(t + TB);
     const int nb = min(TB, t1 - t);
-    for (int tk = 0; tk < nb; ++tk) {
-      const float gi = gate_s[2 * tk], gf = gate_s[2 * tk + 1];
-      const float mn = fmaxf(gf + m, gi);
-      const float a = expf(gf + m - mn), bb = expf(gi - mn);
-      m = mn;
-      const float4* qp = reinterpret_cast<const float4*>(qk_s + (size_t)(tk * 2) * DP + d0);
-      const float4* kp = reinterpret_cast<const float4*>(qk_s + (size_t)(tk * 2 + 1) * DP + d0);
-      const float4 q0 = qp[0], q1 = qp[1], k0 = kp[0], k1 = kp[1];
-      const float q[MM_KPT] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-      const float k[MM_KPT] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-      const float bv = bb * v_s[tk * CPG + cw];
-      float num = 0.f, nq = 0.f;
+    for (int tk0 = 0; tk0 < nb; tk0 += UN) {
+      float a[UN], bv[UN], bb[UN], em[UN], num[UN], nq[UN];
+      // the gates' chain: additions and maxima only; the exponentials hang off it
 #pragma unroll
-      for (int j = 0; j < MM_KPT; ++j) {
-        S[j] = fmaf(a, S[j], k[j] * bv);
-        num = fmaf(S[j], q[j], num);
-        nn[j] = fmaf(a, nn[j], bb * k[j]);
-        nq = fmaf(nn[j], q[j], nq);
+      for (int u = 0; u < UN; ++u) {
+        const bool on = tk0 + u < nb;
+        const float gi = gate_s[2 * (tk0 + u)], gf = gate_s[2 * (tk0 + u) + 1];
+        const float mn = fmaxf(gf + m, gi);
+        a[u] = on ? expf(gf + m - mn) : 1.f;
+        bb[u] = on ? expf(gi - mn) : 0.f;
+        m = on ? mn : m;
+        em[u] = expf(-m);
+        bv[u] = bb[u] * v_s[(tk0 + u) * CPG + cw];
       }
 #pragma unroll
-      for (int o = TPC / 2; o > 0; o >>= 1) {
-        num += __shfl_xor(num, o, NS_WAVE);
-        nq += __shfl_xor(nq, o, NS_WAVE);
+      for (int u = 0; u < UN; ++u) {
+        const float4* qp = reinterpret_cast<const float4*>(qk_s + (size_t)((tk0 + u) * 2) * DP + d0);
+        const float4* kp = reinterpret_cast<const float4*>(qk_s + (size_t)((tk0 + u) * 2 + 1) * DP + d0);
+        const float4 q0 = qp[0], q1 = qp[1], k0 = kp[0], k1 = kp[1];
+        const float q[MM_KPT] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        const float k[MM_KPT] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+        float p0 = 0.f, p1 = 0.f, r0 = 0.f, r1 = 0.f;  // two partial sums each: shorter chains
+#pragma unroll
+        for (int j = 0; j < MM_KPT; j += 2) {
+          S[j] = fmaf(a[u], S[j], k[j] * bv[u]);
+          S[j + 1] = fmaf(a[u], S[j + 1], k[j + 1] * bv[u]);
+          p0 = fmaf(S[j], q[j], p0);
+          p1 = fmaf(S[j + 1], q[j + 1], p1);
+          nn[j] = fmaf(a[u], nn[j], bb[u] * k[j]);
+          nn[j + 1] = fmaf(a[u], nn[j + 1], bb[u] * k[j + 1]);
+          r0 = fmaf(nn[j], q[j], r0);
+          r1 = fmaf(nn[j + 1], q[j + 1], r1);
+        }
+        num[u] = p0 + p1, nq[u] = r0 + r1;
       }
-      if (s == 0 && col_ok) p.out[(size_t)(t + tk) * H * E + (size_t)h * E + col] = num / (fmaxf(fabsf(nq), expf(-m)) + p.den_eps);
+#pragma unroll
+      for (int u = 0; u < UN; ++u) num[u] = group_sum<TPC>(num[u]), nq[u] = group_sum<TPC>(nq[u]);
+      if (s == 0 && col_ok) {
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+          if (tk0 + u < nb) p.out[(size_t)(t + tk0 + u) * H * E + (size_t)h * E + col] = num[u] / (fmaxf(fabsf(nq[u]), em[u]) + p.den_eps);
+      }
     }
     __syncthreads();
     if (t + TB < t1) stage();
