@@ -245,7 +245,7 @@ extern "C" int ns_whole_norm_kv_write(void* qkv, int stride, const void* bias, c
 // ------------------------------------------------------------------------------------------------
 // Queries and keys with biases, an RMS norm per head whose weight [hd] all heads share, and a rotation of the head's first
 // ``rot`` channels; optionally the key projection's raw output (bias added, no norm, no rotation) is stored as the values.
-// One workgroup a token, a wave a head in turn.  A row of ``qkv`` is [q heads | k heads | v heads] (no v part if
+// A workgroup a token (few tokens: several, each with its share of the heads), a wave a head in turn.  A row of ``qkv`` is [q heads | k heads | v heads] (no v part if
 // ``v_is_k``); q is normed and rotated in place, k and v go into the token's slot of their pages.  All of it in 32-bit.
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_rope_kv_write_kernel(
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(256) void head_norm_rope_kv_write_kernel(
   const int page = block_table[(size_t)token_req[t] * table_stride + pos / page_size];
   const int slot = pos % page_size;
   const int half = form.rot / 2;
-  for (int h = wave; h < heads + kv_heads; h += waves) {
+  for (int h = blockIdx.y * waves + wave; h < heads + kv_heads; h += waves * gridDim.y) {
     const bool is_q = h < heads;
     const int at = h * hd;  // q heads and k heads follow each other in the row
     const T* w = is_q ? qw : kw;
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(256) void head_norm_rope_kv_write_kernel(
         kd[c] = from_f<T>(v);
     }
   }
-  if (!v_is_k) {
+  if (!v_is_k && blockIdx.y == 0) {
     const int nq = heads * hd, nk = kv_heads * hd, nv = kv_heads * vd;
     for (int i = threadIdx.x; i < nv; i += blockDim.x) {
       const float v = to_f(row[nq + nk + i]) + (bias ? to_f(bias[nq + nk + i]) : 0.f);
@@ -317,11 +317,15 @@ extern "C" int ns_head_norm_rope_kv_write(void* qkv, int stride, const void* bia
   if (v_is_k && vd != hd) return NS_ERR_BAD_ARG;
   if (rot > 0 && !inv_freq) return NS_ERR_BAD_ARG;
   const RopeForm form{rot, interleaved, factor};
+  // few tokens: a wave a head at once, over several workgroups a token
+  const int shares = n_tokens >= 256 ? 1 : (heads + kv_heads + 3) / 4;
+  if (n_tokens > 65535 * 32768 || shares > 65535) return NS_ERR_BAD_ARG;
+  dim3 grid(n_tokens, shares);
   if (dtype == NS_DTYPE_F32)
-    head_norm_rope_kv_write_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, stride, (const float*)bias, (const float*)qw, (const float*)kw,
+    head_norm_rope_kv_write_kernel<float><<<grid, 256, 0, stream>>>((float*)qkv, stride, (const float*)bias, (const float*)qw, (const float*)kw,
         positions, token_req, block_table, table_stride, inv_freq, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, vd, page_size, eps, form, v_is_k);
   else if (dtype == NS_DTYPE_BF16)
-    head_norm_rope_kv_write_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((bf16_t*)qkv, stride, (const bf16_t*)bias, (const bf16_t*)qw, (const bf16_t*)kw,
+    head_norm_rope_kv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)qkv, stride, (const bf16_t*)bias, (const bf16_t*)qw, (const bf16_t*)kw,
         positions, token_req, block_table, table_stride, inv_freq, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, vd, page_size, eps, form, v_is_k);
   else
     return NS_ERR_UNSUPPORTED;

@@ -10,7 +10,7 @@
 #define MOE_MAX_TOP 32
 
 // Two kernels.  Logits: a workgroup takes ROUTE_TOK tokens and four experts, a wave an expert: it reads the expert's row
-// once (16 bytes a lane a load where the sizes allow) for all of its tokens.  Choice: a thread a token.
+// once (16 bytes a lane a load where the sizes allow) for all of its tokens.  Choice: a wave a token.
 #define ROUTE_TOK 8
 template <typename T>
 __global__ __launch_bounds__(256) void moe_logits_kernel(const T* __restrict__ h, int h_stride, const float* __restrict__ wr,
@@ -50,33 +50,43 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(const T* __restrict__ h
   }
 }
 
+// A wave a token: the logits in LDS, every lane looks through its share for the largest one not yet taken, the lanes'
+// candidates meet by lane exchange (the larger value wins, the lower index among equals; what is no number counts as
+// minus infinity, so a row of anything still chooses ``top`` different experts).
 __global__ __launch_bounds__(64) void moe_choose_kernel(const float* __restrict__ z, int* __restrict__ sel, float* __restrict__ wt, int n,
                                                         int experts, int top) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n) return;
-  const float* zt = z + (size_t)t * experts;
-  int idx[MOE_MAX_TOP];
-  float val[MOE_MAX_TOP];
+  __shared__ float zs[MOE_MAX_EXPERTS];
+  __shared__ unsigned char taken[MOE_MAX_EXPERTS];
+  const int t = blockIdx.x, lane = threadIdx.x;
+  for (int e = lane; e < experts; e += NS_WAVE) {
+    const float v = z[(size_t)t * experts + e];
+    zs[e] = v == v ? v : -INFINITY;
+    taken[e] = 0;
+  }
+  __syncthreads();
+  float largest = 0.f, sum = 0.f, mine = 0.f;  // lane k keeps the k-th chosen value
+  int mine_idx = 0;
   for (int k = 0; k < top; ++k) {
     int best = -1;
     float bv = -INFINITY;
-    for (int e = 0; e < experts; ++e) {
-      bool taken = false;
-      for (int j = 0; j < k; ++j) taken |= idx[j] == e;
-      const float v = zt[e];
-      if (!taken && (best < 0 || v > bv)) best = e, bv = v;
+    for (int e = lane; e < experts; e += NS_WAVE)
+      if (!taken[e] && (best < 0 || zs[e] > bv)) best = e, bv = zs[e];
+#pragma unroll
+    for (int o = NS_WAVE / 2; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, NS_WAVE);
+      const int oi = __shfl_xor(best, o, NS_WAVE);
+      if (oi >= 0 && (best < 0 || ov > bv || (ov == bv && oi < best))) best = oi, bv = ov;
     }
-    idx[k] = best, val[k] = bv;
+    if (lane == 0) taken[best] = 1;
+    if (k == 0) largest = bv;
+    const float w = expf(bv - largest);
+    sum += w;
+    if (lane == k % NS_WAVE && k < NS_WAVE) mine = w, mine_idx = best;
+    __syncthreads();
   }
-  float sum = 0.f;
-  const float largest = val[0];
-  for (int k = 0; k < top; ++k) {
-    val[k] = expf(val[k] - largest);
-    sum += val[k];
-  }
-  for (int k = 0; k < top; ++k) {
-    sel[(size_t)t * top + k] = idx[k];
-    wt[(size_t)t * top + k] = val[k] / sum;
+  if (lane < top) {
+    sel[(size_t)t * top + lane] = mine_idx;
+    wt[(size_t)t * top + lane] = mine / sum;
   }
 }
 
@@ -94,7 +104,7 @@ extern "C" int ns_moe_route(const void* h, int h_stride, const float* wr, const 
     moe_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)h, h_stride, wr, br, z, n, W, experts, vec);
   else
     return NS_ERR_UNSUPPORTED;
-  moe_choose_kernel<<<(n + 63) / 64, 64, 0, stream>>>(z, sel, wt, n, experts, top);
+  moe_choose_kernel<<<n, 64, 0, stream>>>(z, sel, wt, n, experts, top);
   return ns_launch_status();
 }
 
@@ -212,19 +222,23 @@ extern "C" int ns_moe_expert_rows(const void* h, int h_stride, const void* wg, c
 
 // ------------------------------------------------------------------------------------------------ many rows
 // Steps of many rows (bfloat16): the (token, chosen expert) pairs are sorted by expert on the device, and every expert's
-// pairs are cut into tiles of 64 rows.  A workgroup takes one tile and 64 output channels and multiplies on the matrix
-// cores (v_mfma_f32_16x16x32_bf16): its four waves own 32 x 32 each, operands come through LDS in pieces of 64 along K,
+// pairs are cut into tiles of 128 rows.  A workgroup takes one tile and 128 output channels and multiplies on the matrix
+// cores (v_mfma_f32_16x16x32_bf16): its four waves own 64 x 64 each, operands come through LDS in pieces of 64 along K,
 // the next piece is fetched into registers while the current one is multiplied.  The host never learns which experts were
-// chosen: the launch has as many tiles as any choice can need (pairs / 64 + experts), and a tile without rows returns.
+// chosen: the launch has as many tiles as any choice can need (pairs / 128 + experts), and a tile without rows returns.
 //   first:  rows gathered from h by the sorted pairs; gate and up matrices in the same pass; act [pairs sorted][ff] in bfloat16
 //   second: act times the down matrix; out [tokens][top][W] in 32-bit, each row back at its pair and times its weight
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
-#define MG_TM 64
-#define MG_TN 64
+#define MG_TM 128
+#define MG_TN 128
 #define MG_KC 64
 #define MG_LD (MG_KC + 8)  // bfloat16 values between two rows of a staged tile (padded: neighbouring rows start in other banks)
+#define MG_RI (MG_TM / 32)  // 16-row blocks of a wave's 64 x 64 (the four waves are 2 x 2)
+#define MG_CJ (MG_TN / 32)
+#define MG_FA (MG_TM / 32)  // pieces of 8 values that a thread fetches of a staged tile of MG_TM rows (256 threads, 8 pieces a row)
+#define MG_FB (MG_TN / 32)
 
 __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ sel, int pairs, int experts, int* __restrict__ perm,
                                                         int* __restrict__ tile_e, int* __restrict__ tile_r0, int* __restrict__ tile_rows,
@@ -267,46 +281,55 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16_t* __restrict
   const int wm = wave / 2, wn = wave % 2;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  // the two pieces (8 values along K) of each staged tile that this thread fetches: rows tid / 8 and tid / 8 + 32, piece tid % 8
+  // the pieces (8 values along K) of each staged tile that this thread fetches: rows tid / 8 + 32 i, piece tid % 8
   const int kp = (tid % 8) * 8;
-  const bf16_t* arow[2];
-  const bf16_t* brow0[2];
-  const bf16_t* brow1[2];
+  const bf16_t* arow[MG_FA];
+  const bf16_t* brow0[MG_FB];
+  const bf16_t* brow1[MG_FB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < MG_FA; ++i) {
     const int row = tid / 8 + 32 * i;
     const int slot = r0 + row;
     arow[i] = row < rows ? A + (size_t)(DUAL ? perm[slot] / top : slot) * a_stride : nullptr;
-    const int col = n0 + row;
+  }
+#pragma unroll
+  for (int i = 0; i < MG_FB; ++i) {
+    const int col = n0 + tid / 8 + 32 * i;
     brow0[i] = col < N ? B0 + ((size_t)e * N + col) * K : nullptr;
     brow1[i] = (DUAL && col < N) ? B1 + ((size_t)e * N + col) * K : nullptr;
   }
-  bf16x8 pa[2], pb0[2], pb1[2];
+  bf16x8 pa[MG_FA], pb0[MG_FB], pb1[MG_FB];
   auto fetch = [&](int k0) {
     const bool ok = k0 + kp < K;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      pa[i] = (ok && arow[i]) ? *reinterpret_cast<const bf16x8*>(arow[i] + k0 + kp) : zero;
+    for (int i = 0; i < MG_FA; ++i) pa[i] = (ok && arow[i]) ? *reinterpret_cast<const bf16x8*>(arow[i] + k0 + kp) : zero;
+#pragma unroll
+    for (int i = 0; i < MG_FB; ++i) {
       pb0[i] = (ok && brow0[i]) ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(brow0[i] + k0 + kp)) : zero;
       if (DUAL) pb1[i] = (ok && brow1[i]) ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(brow1[i] + k0 + kp)) : zero;
     }
   };
   auto stage = [&]() {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < MG_FA; ++i) *reinterpret_cast<bf16x8*>(As + (tid / 8 + 32 * i) * MG_LD + kp) = pa[i];
+#pragma unroll
+    for (int i = 0; i < MG_FB; ++i) {
       const int at = (tid / 8 + 32 * i) * MG_LD + kp;
-      *reinterpret_cast<bf16x8*>(As + at) = pa[i];
       *reinterpret_cast<bf16x8*>(Bs + at) = pb0[i];
       if (DUAL) *reinterpret_cast<bf16x8*>(Bs + MG_TN * MG_LD + at) = pb1[i];
     }
   };
 
-  f32x4 acc0[2][2], acc1[2][2];
+  f32x4 acc0[MG_RI][MG_CJ], acc1[DUAL ? MG_RI : 1][DUAL ? MG_CJ : 1];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MG_RI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) acc0[i][j] = f32x4{0.f, 0.f, 0.f, 0.f}, acc1[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < MG_CJ; ++j) {
+      acc0[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (DUAL) acc1[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
 
+  const int a_at = (MG_TM / 2 * wm + r) * MG_LD + 8 * g, b_at = (MG_TN / 2 * wn + r) * MG_LD + 8 * g;
   fetch(0);
   for (int k0 = 0; k0 < K; k0 += MG_KC) {
     stage();
@@ -314,17 +337,18 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16_t* __restrict
     if (k0 + MG_KC < K) fetch(k0 + MG_KC);
 #pragma unroll
     for (int ks = 0; ks < MG_KC; ks += 32) {
-      bf16x8 af[2], bf0[2], bf1[2];
+      bf16x8 af[MG_RI], bf0[MG_CJ], bf1[MG_CJ];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        af[i] = *reinterpret_cast<const bf16x8*>(As + (32 * wm + 16 * i + r) * MG_LD + ks + 8 * g);
-        bf0[i] = *reinterpret_cast<const bf16x8*>(Bs + (32 * wn + 16 * i + r) * MG_LD + ks + 8 * g);
-        if (DUAL) bf1[i] = *reinterpret_cast<const bf16x8*>(Bs + MG_TN * MG_LD + (32 * wn + 16 * i + r) * MG_LD + ks + 8 * g);
+      for (int i = 0; i < MG_RI; ++i) af[i] = *reinterpret_cast<const bf16x8*>(As + a_at + 16 * i * MG_LD + ks);
+#pragma unroll
+      for (int j = 0; j < MG_CJ; ++j) {
+        bf0[j] = *reinterpret_cast<const bf16x8*>(Bs + b_at + 16 * j * MG_LD + ks);
+        if (DUAL) bf1[j] = *reinterpret_cast<const bf16x8*>(Bs + MG_TN * MG_LD + b_at + 16 * j * MG_LD + ks);
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < MG_RI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < MG_CJ; ++j) {
           acc0[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf0[j], acc0[i][j], 0, 0, 0);
           if (DUAL) acc1[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf1[j], acc1[i][j], 0, 0, 0);
         }
@@ -333,17 +357,17 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16_t* __restrict
   }
   // element q of a lane's sums is row 4 g + q of the 16 x 16 block, column r
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MG_RI; ++i)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int row = 32 * wm + 16 * i + 4 * g + q;
+      const int row = MG_TM / 2 * wm + 16 * i + 4 * g + q;
       if (row >= rows) continue;
       const int slot = r0 + row;
       const int pair = DUAL ? 0 : perm[slot];
       const float share = DUAL ? 0.f : wt[pair];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int col = n0 + 32 * wn + 16 * j + r;
+      for (int j = 0; j < MG_CJ; ++j) {
+        const int col = n0 + MG_TN / 2 * wn + 16 * j + r;
         if (col >= N) continue;
         if (DUAL)
           act_out[(size_t)slot * N + col] = from_f<bf16_t>(clipped_glu(round_to<bf16_t>(acc0[i][j][q]), round_to<bf16_t>(acc1[i][j][q]), limit, alpha));
@@ -366,12 +390,12 @@ extern "C" int ns_moe_expert_groups(const void* h, int h_stride, const void* wg,
   const long long pairs = (long long)n * top;
   if (pairs > (1 << 24)) return NS_ERR_UNSUPPORTED;
   const int tiles = ns_moe_group_tiles((int)pairs, experts);
-  if (tiles > 65535) return NS_ERR_UNSUPPORTED;
   int* perm = ints;
   int* tile_e = ints + pairs;
   int* tile_r0 = tile_e + tiles;
   int* tile_rows = tile_r0 + tiles;
   moe_sort_kernel<<<1, 1024, 0, stream>>>(sel, (int)pairs, experts, perm, tile_e, tile_r0, tile_rows, tiles);
+  if (tiles > 65535) return NS_ERR_UNSUPPORTED;
   dim3 g1((ff + MG_TN - 1) / MG_TN, tiles), g2((W + MG_TN - 1) / MG_TN, tiles);
   moe_group_kernel<true><<<g1, 256, 0, stream>>>((const bf16_t*)h, h_stride, (const bf16_t*)wg, (const bf16_t*)wu, perm, tile_e, tile_r0, tile_rows,
                                                   (bf16_t*)act, nullptr, nullptr, ff, W, top, limit, alpha);
