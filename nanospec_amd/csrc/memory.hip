@@ -8,14 +8,17 @@
 // result of one stacked product), in the model's precision; everything from there on is 32-bit.
 //
 // A column of S never meets another column, so a wave owns 64 / TPC columns and the TPC lanes of a column hold 8 key
-// channels each; their partial sums meet through the vector unit's lane permutations (``group_sum``).  Every column's lanes also carry n (the same in all columns),
-// so no wave waits for another.  A workgroup is four waves that share the staged operands: the next block of tokens is
-// fetched into registers while the current block is worked through from LDS.
+// channels each; their partial sums meet through the vector unit's lane permutations (``group_sum``).  n is one more column
+// of S, the one whose value is 1 for every token: one more workgroup a head carries it, and what it writes per token is the
+// denominator max(|n . q|, exp(-m')) + den_eps.  The kernel leaves S^T q and the denominators; whoever reads the read-out
+// divides (``gated_rms`` does, as it reads a head).  A workgroup is four waves that share the staged operands: the next
+// block of tokens is fetched into registers while the current block is worked through from LDS, and four tokens are
+// worked through together: only m, S and n pass from token to token.
 //
 // What a request keeps between steps lies in its state slot: S as [H][E][D] (a column's key channels contiguous), then
-// one copy of n per workgroup of a head, [H][B][D], then m likewise, [H][B], with B = ``ns_memory_blocks(D, E)`` the
-// workgroups that share a head's columns: a workgroup reads and writes only its own copy, so none can read what another
-// has already written for the next step.
+// room for n per workgroup of a head, [H][B][D] (the last workgroup's is the one in use), then m per workgroup, [H][B],
+// with B = ``ns_memory_blocks(D, E)`` the workgroups of a head: each reads and writes only its own copy of m, so none can
+// read what another has already written for the next step.
 #include "common.h"
 
 #define MM_KPT 8  // key channels a lane holds of its column
@@ -52,7 +55,8 @@ struct MemoryParams {
   long long state_stride;
   const int* qo_indptr;
   const int* state_slots;
-  float* out;  // [tokens][H * E]
+  float* out;  // [tokens][H * E]: S^T q, not yet divided
+  float* den;  // [tokens][H]: max(|n . q|, exp(-m)) + den_eps
   int H, D, E;
   float cap, q_scale, den_eps;
   int vec_ok;  // 8 channels of q and k can be fetched with one aligned vector load
@@ -77,7 +81,10 @@ __global__ __launch_bounds__(MM_THREADS) void memory_scan_kernel(const MemoryPar
   if (t1 <= t0) return;
   const int H = p.H, D = p.D, E = p.E;
   const int s = lane % TPC, cw = wave * CPW + lane / TPC, col = blockIdx.x * CPG + cw, d0 = s * MM_KPT;
-  const bool col_ok = col < E;
+  // the last workgroup of a head carries n as one more column of S whose value is 1 for every token: its first column's
+  // lanes hold n where the others hold a column of S, and what it writes is the denominator
+  const bool nblock = blockIdx.x == gridDim.x - 1;
+  const bool col_ok = !nblock && col < E, n_lane = nblock && cw == 0;
   const T* proj = (const T*)p.proj;
   float* st = p.state + (long long)p.state_slots[b] * p.state_stride;
   float* st_S = st + ((size_t)h * E + (col_ok ? col : 0)) * D;
@@ -85,12 +92,11 @@ __global__ __launch_bounds__(MM_THREADS) void memory_scan_kernel(const MemoryPar
   float* st_n = st + (size_t)H * E * D + ((size_t)h * B + blockIdx.x) * D;
   float* st_m = st + (size_t)H * E * D + (size_t)H * B * D + (size_t)h * B + blockIdx.x;
 
-  float S[MM_KPT], nn[MM_KPT];
+  float S[MM_KPT];
 #pragma unroll
   for (int j = 0; j < MM_KPT; ++j) {
     const bool ok = d0 + j < D;
-    S[j] = (ok && col_ok) ? st_S[d0 + j] : 0.f;
-    nn[j] = ok ? st_n[d0 + j] : 0.f;
+    S[j] = (ok && col_ok) ? st_S[d0 + j] : ((ok && n_lane) ? st_n[d0 + j] : 0.f);
   }
   float m = *st_m;
   const float bias_i = p.gate_bias_i ? p.gate_bias_i[h] : 0.f, bias_f = p.gate_bias_f ? p.gate_bias_f[h] : 0.f;
@@ -119,7 +125,10 @@ __global__ __launch_bounds__(MM_THREADS) void memory_scan_kernel(const MemoryPar
 #pragma unroll
     for (int i = 0; i < VPER; ++i) {
       const int idx = tid + i * MM_THREADS, tk = idx / CPG, c = blockIdx.x * CPG + idx % CPG;
-      vpre[i] = (idx < VALS && t + tk < t1 && c < E) ? to_f(proj[(size_t)(t + tk) * p.stride + p.v_off + (size_t)h * E + c]) : 0.f;
+      if (nblock)
+        vpre[i] = idx % CPG == 0 ? 1.f : 0.f;
+      else
+        vpre[i] = (idx < VALS && t + tk < t1 && c < E) ? to_f(proj[(size_t)(t + tk) * p.stride + p.v_off + (size_t)h * E + c]) : 0.f;
     }
     if (tid < 2 * TB) {
       const int tk = tid / 2, which = tid % 2;
@@ -157,7 +166,7 @@ __global__ __launch_bounds__(MM_THREADS) void memory_scan_kernel(const MemoryPar
     if (t + TB < t1) fetch(t + TB);
     const int nb = min(TB, t1 - t);
     for (int tk0 = 0; tk0 < nb; tk0 += UN) {
-      float a[UN], bv[UN], bb[UN], em[UN], num[UN], nq[UN];
+      float a[UN], bv[UN], em[UN], num[UN];
       // the gates' chain: additions and maxima only; the exponentials hang off it
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
@@ -165,10 +174,10 @@ __global__ __launch_bounds__(MM_THREADS) void memory_scan_kernel(const MemoryPar
         const float gi = gate_s[2 * (tk0 + u)], gf = gate_s[2 * (tk0 + u) + 1];
         const float mn = fmaxf(gf + m, gi);
         a[u] = on ? expf(gf + m - mn) : 1.f;
-        bb[u] = on ? expf(gi - mn) : 0.f;
+        const float bb = on ? expf(gi - mn) : 0.f;
         m = on ? mn : m;
-        em[u] = expf(-m);
-        bv[u] = bb[u] * v_s[(tk0 + u) * CPG + cw];
+        em[u] = nblock ? expf(-m) : 0.f;
+        bv[u] = bb * v_s[(tk0 + u) * CPG + cw];
       }
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
@@ -177,26 +186,27 @@ __global__ __launch_bounds__(MM_THREADS) void memory_scan_kernel(const MemoryPar
         const float4 q0 = qp[0], q1 = qp[1], k0 = kp[0], k1 = kp[1];
         const float q[MM_KPT] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
         const float k[MM_KPT] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-        float p0 = 0.f, p1 = 0.f, r0 = 0.f, r1 = 0.f;  // two partial sums each: shorter chains
+        float p0 = 0.f, p1 = 0.f;  // two partial sums: shorter chains
 #pragma unroll
         for (int j = 0; j < MM_KPT; j += 2) {
           S[j] = fmaf(a[u], S[j], k[j] * bv[u]);
           S[j + 1] = fmaf(a[u], S[j + 1], k[j + 1] * bv[u]);
           p0 = fmaf(S[j], q[j], p0);
           p1 = fmaf(S[j + 1], q[j + 1], p1);
-          nn[j] = fmaf(a[u], nn[j], bb[u] * k[j]);
-          nn[j + 1] = fmaf(a[u], nn[j + 1], bb[u] * k[j + 1]);
-          r0 = fmaf(nn[j], q[j], r0);
-          r1 = fmaf(nn[j + 1], q[j + 1], r1);
         }
-        num[u] = p0 + p1, nq[u] = r0 + r1;
+        num[u] = p0 + p1;
       }
 #pragma unroll
-      for (int u = 0; u < UN; ++u) num[u] = group_sum<TPC>(num[u]), nq[u] = group_sum<TPC>(nq[u]);
-      if (s == 0 && col_ok) {
+      for (int u = 0; u < UN; ++u) num[u] = group_sum<TPC>(num[u]);
+      if (s == 0 && (col_ok || n_lane)) {
 #pragma unroll
         for (int u = 0; u < UN; ++u)
-          if (tk0 + u < nb) p.out[(size_t)(t + tk0 + u) * H * E + (size_t)h * E + col] = num[u] / (fmaxf(fabsf(nq[u]), em[u]) + p.den_eps);
+          if (tk0 + u < nb) {
+            if (n_lane)
+              p.den[(size_t)(t + tk0 + u) * H + h] = fmaxf(fabsf(num[u]), em[u]) + p.den_eps;
+            else
+              p.out[(size_t)(t + tk0 + u) * H * E + (size_t)h * E + col] = num[u];
+          }
       }
     }
     __syncthreads();
@@ -207,7 +217,7 @@ __global__ __launch_bounds__(MM_THREADS) void memory_scan_kernel(const MemoryPar
   for (int j = 0; j < MM_KPT; ++j) {
     if (d0 + j < D) {
       if (col_ok) st_S[d0 + j] = S[j];
-      if (cw == 0) st_n[d0 + j] = nn[j];
+      if (n_lane) st_n[d0 + j] = S[j];
     }
   }
   if (tid == 0) *st_m = m;
@@ -219,7 +229,7 @@ static int memory_scan_launch(const MemoryParams& p, int n_reqs, hipStream_t str
   while (tpc * MM_KPT < p.D) tpc *= 2;
   if (tpc > NS_WAVE) return NS_ERR_UNSUPPORTED;
   const int cpg = MM_WAVES * NS_WAVE / tpc;
-  dim3 grid((p.E + cpg - 1) / cpg, p.H, n_reqs);
+  dim3 grid((p.E + cpg - 1) / cpg + 1, p.H, n_reqs);  // one more workgroup a head: the one that carries n
   switch (tpc) {
     case 1: memory_scan_kernel<T, 1><<<grid, MM_THREADS, 0, stream>>>(p); break;
     case 2: memory_scan_kernel<T, 2><<<grid, MM_THREADS, 0, stream>>>(p); break;
@@ -232,24 +242,24 @@ static int memory_scan_launch(const MemoryParams& p, int n_reqs, hipStream_t str
   return ns_launch_status();
 }
 
-// workgroups that share the columns of one head (each keeps a copy of n and m in the state)
+// workgroups of one head: those that share its columns and the one that carries n (each keeps a copy of m, and room for n, in the state)
 extern "C" int ns_memory_blocks(int D, int E) {
   int tpc = 1;
   while (tpc * MM_KPT < D) tpc *= 2;
   if (tpc > NS_WAVE) return -1;
   const int cpg = MM_WAVES * NS_WAVE / tpc;
-  return (E + cpg - 1) / cpg;
+  return (E + cpg - 1) / cpg + 1;
 }
 
 extern "C" int ns_memory_scan(const void* proj, int stride, int q_off, int k_off, int v_off, int i_off, int f_off, const float* gate_bias_i,
                               const float* gate_bias_f, float* state, long long state_stride, const int* qo_indptr, const int* state_slots,
-                              float* out, int n_reqs, int H, int D, int E, float cap, float q_scale, float den_eps, int dtype, hipStream_t stream) {
+                              float* out, float* den, int n_reqs, int H, int D, int E, float cap, float q_scale, float den_eps, int dtype, hipStream_t stream) {
   if (n_reqs <= 0 || n_reqs > 65535 || H <= 0 || H > 65535 || D <= 0 || E <= 0 || !(cap > 0.f)) return NS_ERR_BAD_ARG;
   const int blocks = ns_memory_blocks(D, E);
   if (blocks < 0) return NS_ERR_UNSUPPORTED;
   if (state_stride < (long long)H * E * D + (long long)H * blocks * (D + 1)) return NS_ERR_BAD_ARG;
   MemoryParams p{proj, stride, q_off, k_off, v_off, i_off, f_off, gate_bias_i, gate_bias_f, state, state_stride, qo_indptr, state_slots,
-                 out, H, D, E, cap, q_scale, den_eps, 0};
+                 out, den, H, D, E, cap, q_scale, den_eps, 0};
   const size_t elem = dtype == NS_DTYPE_F32 ? 4 : 2;
   p.vec_ok = D % 8 == 0 && stride % 8 == 0 && q_off % 8 == 0 && k_off % 8 == 0 && ((uintptr_t)proj % (8 * elem)) == 0;
   if (dtype == NS_DTYPE_F32) return memory_scan_launch<float>(p, n_reqs, stream);

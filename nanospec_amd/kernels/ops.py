@@ -1080,7 +1080,8 @@ MOE_MAX_EXPERTS, MOE_MAX_TOP = 1024, 32
 
 
 def memory_blocks(key_dim: int, value_dim: int) -> int:
-    """Workgroups that share the columns of one head in ``memory_scan``: the state keeps a copy of n and m for each."""
+    """Workgroups of one head in ``memory_scan`` (those that share its columns, and the one that carries n): the state keeps
+    a copy of m, and room for n, for each."""
     b = int(build.core().ns_memory_blocks(c_int(key_dim), c_int(value_dim)))
     if b < 0:
         raise KernelRefused(f"memory_scan takes key sizes up to 512, not {key_dim}")
@@ -1094,20 +1095,21 @@ def memory_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
 
 def memory_scan(proj: torch.Tensor, offsets: tuple[int, int, int, int, int], gate_bias_i: torch.Tensor | None, gate_bias_f: torch.Tensor | None,
                 state: torch.Tensor, qo_indptr, state_slots, heads: int, key_dim: int, value_dim: int, cap: float, q_scale: float,
-                out: torch.Tensor, den_eps: float = 1e-6) -> torch.Tensor:
+                out: torch.Tensor, den: torch.Tensor, den_eps: float = 1e-6) -> torch.Tensor:
     """The matrix memory's recurrence over every request's tokens of the step, in order (``csrc/memory.hip``).  A row of
     ``proj`` holds q and k [heads * key_dim], v [heads * value_dim] and the two gate inputs [heads] at the column
-    ``offsets`` (q, k, v, input gate, forget gate); ``state`` float32 [slots, >= memory_state_floats]; ``out`` float32
-    [tokens, heads * value_dim]."""
-    _gpu(proj, state, qo_indptr, state_slots, out, gate_bias_i, gate_bias_f)
-    _f32(out, "out"), _i32(qo_indptr, "qo_indptr"), _i32(state_slots, "state_slots")
+    ``offsets`` (q, k, v, input gate, forget gate); ``state`` float32 [slots, >= memory_state_floats].  ``out`` float32
+    [tokens, heads * value_dim] receives S^T q and ``den`` float32 [tokens, heads] the denominators max(|n . q|, exp(-m)) +
+    den_eps: the read-out is out / den (``gated_rms`` divides as it reads)."""
+    _gpu(proj, state, qo_indptr, state_slots, out, den, gate_bias_i, gate_bias_f)
+    _f32(out, "out"), _f32(den, "den"), _i32(qo_indptr, "qo_indptr"), _i32(state_slots, "state_slots")
     n = proj.shape[0]
     q_off, k_off, v_off, i_off, f_off = offsets
     if proj.dim() != 2 or proj.stride(1) != 1 or max(q_off, k_off) + heads * key_dim > proj.shape[1] or v_off + heads * value_dim > proj.shape[1] \
             or max(i_off, f_off) + heads > proj.shape[1]:
         raise KernelRefused("memory_scan: the row does not hold q, k, v and the gates at the given columns")
-    if out.shape != (n, heads * value_dim):
-        raise KernelRefused(f"memory_scan: out must be float32 [{n}, {heads * value_dim}]")
+    if out.shape != (n, heads * value_dim) or not out.is_contiguous() or den.shape != (n, heads) or not den.is_contiguous():
+        raise KernelRefused(f"memory_scan: out must be float32 [{n}, {heads * value_dim}] and den float32 [{n}, {heads}]")
     if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < memory_state_floats(heads, key_dim, value_dim):
         raise KernelRefused("memory_scan: state is float32 [slots, words] with room for S, n and m")
     for t in (gate_bias_i, gate_bias_f):
@@ -1118,7 +1120,7 @@ def memory_scan(proj: torch.Tensor, offsets: tuple[int, int, int, int, int], gat
         raise KernelRefused("memory_scan: one state slot per request")
     _check(build.core().ns_memory_scan(_ptr(proj), c_int(proj.stride(0)), c_int(q_off), c_int(k_off), c_int(v_off), c_int(i_off), c_int(f_off),
                                        _ptr(gate_bias_i), _ptr(gate_bias_f), _ptr(state), ctypes.c_longlong(state.stride(0)), _ptr(qo_indptr),
-                                       _ptr(state_slots), _ptr(out), c_int(reqs), c_int(heads), c_int(key_dim), c_int(value_dim), c_float(cap),
+                                       _ptr(state_slots), _ptr(out), _ptr(den), c_int(reqs), c_int(heads), c_int(key_dim), c_int(value_dim), c_float(cap),
                                        c_float(q_scale), c_float(den_eps), c_int(_dtype_code(proj)), _stream()), "memory_scan")
     return out
 
@@ -1458,19 +1460,21 @@ def delta_scan(qkv: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, state: to
     return out
 
 
-def gated_rms(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, out: torch.Tensor) -> torch.Tensor:
-    """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight * sigmoid(gate[t, h, :]); ``o`` float32 [tokens,
-    heads * E], ``weight`` float32 [E] (all heads share it) or [heads * E], ``gate`` (may be a column slice) and ``out`` in the
-    model's dtype."""
+def gated_rms(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, out: torch.Tensor,
+              den: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t, h, :] = x / sqrt(mean(x^2) + eps) * weight * sigmoid(gate[t, h, :]) with x = o[t, h, :], or o[t, h, :] /
+    den[t, h] if ``den`` (float32 [tokens, heads]) is given; ``o`` float32 [tokens, heads * E], ``weight`` float32 [E] (all
+    heads share it) or [heads * E], ``gate`` (may be a column slice) and ``out`` in the model's dtype."""
     _f32(o, "o"), _f32(weight, "weight")
-    _gpu(gate, out)
+    _gpu(gate, out, den)
     n, width = o.shape
     if (width % heads or weight.numel() not in (width // heads, width) or gate.shape[0] != n or gate.shape[1] < width or gate.stride(1) != 1
-            or out.shape != (n, width) or not out.is_contiguous() or out.dtype != gate.dtype):
+            or out.shape != (n, width) or not out.is_contiguous() or out.dtype != gate.dtype
+            or (den is not None and (_f32(den, "den").shape != (n, heads) or not den.is_contiguous()))):
         raise KernelRefused("gated_rms: operands do not fit heads and value size")
     per_head = width // heads if (weight.numel() == width and heads > 1) else 0
-    _check(build.core().ns_gated_rms(_ptr(out), _ptr(o), _ptr(gate), c_int(gate.stride(0)), _ptr(weight), c_int(per_head), c_int(n), c_int(heads),
-                                     c_int(width // heads), c_float(eps), c_int(_dtype_code(gate)), _stream()), "gated_rms")
+    _check(build.core().ns_gated_rms(_ptr(out), _ptr(o), _ptr(gate), c_int(gate.stride(0)), _ptr(weight), c_int(per_head), _ptr(den), c_int(n),
+                                     c_int(heads), c_int(width // heads), c_float(eps), c_int(_dtype_code(gate)), _stream()), "gated_rms")
     return out
 
 

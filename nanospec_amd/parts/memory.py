@@ -9,7 +9,7 @@ h [tokens, hidden] is the mixer's input; H heads, D key channels, E value channe
 S, n and m start at zero (m at 0, not at minus infinity) and live in 32-bit in the request's state slot.
 
 One product reads h for q, k, v, the output gate and the two gate inputs together (the matrices are stacked at load
-time); gates, recurrence and the gated norm are 32-bit kernels (``csrc/memory.hip``, ``gated_rms`` of ``csrc/delta.hip``).
+time); gates, recurrence (which leaves S^T q and the denominators) and the gated norm (which divides) are 32-bit kernels (``csrc/memory.hip``, ``gated_rms`` of ``csrc/delta.hip``).
 The recurrence walks every request's tokens of the step in order, so portions of prompts, single tokens and padding rows
 (they own the pad slot) need nothing special.
 """
@@ -89,10 +89,12 @@ class MatrixMemory:
         s = self.spec
         n, take = x.shape[0], ctx.arena.take
         proj = self.w_in(x, out=take((n, self.w_in.n), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
+        den = take((n, s.heads), torch.float32)  # the read-out's denominators; the gated norm divides as it reads a head
         o = ops.memory_scan(proj, (0, self.k_at, self.v_at, self.i_at, self.f_at), self.bias_i, self.bias_f, cache.state, ctx.qo_indptr,
                             ctx.state_slots, s.heads, s.key_dim, s.value_dim, s.gate_cap, s.key_dim ** -0.5, den_eps=s.den_eps,
-                            out=take((n, self.vw), torch.float32))
-        gated = ops.gated_rms(o, proj[:, self.g_at : self.g_at + self.vw], self.norm, s.norm_eps, s.heads, out=take((n, self.vw), x.dtype))
+                            out=take((n, self.vw), torch.float32), den=den)
+        gated = ops.gated_rms(o, proj[:, self.g_at : self.g_at + self.vw], self.norm, s.norm_eps, s.heads, out=take((n, self.vw), x.dtype),
+                              den=den)
         return self.w_out(gated, out=out if out is not None else take((n, s.hidden), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
 
 
