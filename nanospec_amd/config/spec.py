@@ -99,6 +99,13 @@ class AttentionSpec:
     head_norm_suffix: str = ".norm"
     # the key projection's raw output (bias added, no norm, no rotation) serves as the values too; the layer has no value matrix
     value_is_key: bool = False
+    # a learned sink: the soft-max's denominator holds one more term exp(sink_h), one stored value per head (the tensor
+    # ``sink_name`` [heads] after the prefix), which has no key and no value and is not scaled
+    sink_name: str = ""
+    # an output gate: the concatenated heads' outputs are multiplied, channel by channel, by sigmoid(W_g h) before the output
+    # projection; W_g [heads * value size, hidden] is the tensor ``gate_name`` after the prefix and reads the mixer's input
+    out_gate: bool = False
+    gate_name: str = "g"
 
     @property
     def v_dim(self) -> int:
@@ -108,16 +115,17 @@ class AttentionSpec:
     def general(self) -> bool:
         return bool(self.value_dim not in (0, self.head_dim) or self.qk_norm_eps is not None or self.score_cap or self.chunk or self.sink
                     or not self.own_kv or self.bias or self.whole_norm_eps is not None or self.slope_exp or self.value_mix
-                    or self.head_norm_eps is not None or self.value_is_key)
+                    or self.head_norm_eps is not None or self.value_is_key or self.sink_name or self.out_gate)
 
 
 @dataclass(frozen=True)
 class LatentAttentionSpec:
     """Soft-max attention whose keys and values come from one cached latent per token.  With h the input:
-    c_q = norm(W_dq h); q = W_uq c_q, per head [dim unrotated | rot rotated];  W_dkv h = [latent | rot]: c = norm(first part),
+    c_q = norm(W_dq h); q = W_uq c_q (``q_rank`` = 0: q = W_uq h, no query latent), per head [dim unrotated | rot rotated];  W_dkv h = [latent | rot]: c = norm(first part),
     the rest is one rotated key part for all heads;  per head k = [W_uk c | rotated part], v = W_uv c;
     score = q . k * softmax_scale over the last ``window`` positions (0: all);  head outputs times sigmoid(W_g h) per head
-    if ``gate``;  then W_o.  The two norms are RMS norms with plain weights.  Only c and the rotated part are cached."""
+    if ``gate``;  then W_o.  The two norms are RMS norms with plain weights.  Only c and the rotated part are cached.
+    ``sink_name``: a learned sink as in ``AttentionSpec`` (one value per head, "" for none)."""
 
     kind: ClassVar[str] = "latent_attention"
     hidden: int
@@ -134,6 +142,7 @@ class LatentAttentionSpec:
     gate: bool = True
     # after the prefix: W_dq, its norm, W_uq, W_dkv, its norm, W_uk, W_uv, W_g, W_o
     names: tuple = ("dq", "dq.norm", "uq", "dkv", "dkv.norm", "uk", "uv", "g", "o")
+    sink_name: str = ""
 
 
 @dataclass(frozen=True)
@@ -180,6 +189,27 @@ class MatrixMemorySpec:
 
 
 @dataclass(frozen=True)
+class RetentionSpec:
+    """Retention: linear attention with one fixed decay per head, no soft-max and no denominator.  With h the input, per
+    head: q = W_q h, k = W_k h [key_dim], v = W_v h [value_dim]; q and k are rotated by their position (``position``), k is
+    then multiplied by ``key_scale``;  S [key_dim, value_dim] starts at zero:
+        S_t = decay_h S_(t-1) + k_t v_t^T;   o_t = S_t^T q_t
+    then o / rms(o) per head (``norm_eps``, no weight), times silu(W_g h), through W_o.  Rotation, decay, state and read-out
+    are 32-bit.  ``names``: q, k, v, the gate, o after the prefix."""
+
+    kind: ClassVar[str] = "retention"
+    hidden: int
+    heads: int
+    key_dim: int
+    value_dim: int
+    decay: tuple[float, ...]  # one per head
+    position: object
+    key_scale: float
+    norm_eps: float
+    names: tuple = ("q", "k", "v", "g", "o")
+
+
+@dataclass(frozen=True)
 class ParallelMixerSpec:
     """Two mixers side by side that read the same input: left_scale * left(h) + right_scale * right(h).  Each keeps what it
     keeps (pages, state); their tensors lie under the two prefixes."""
@@ -195,11 +225,23 @@ class ParallelMixerSpec:
 @dataclass(frozen=True)
 class ClippedGLUSpec:
     """One gated feed-forward with clipped inputs: g = min(W_gate h, limit); u = clamp(W_up h, -limit, limit);
-    W_down (g sigmoid(alpha g) (u + 1)).  No biases."""
+    W_down (g sigmoid(alpha g) (u + shift)).  No biases.  An infinite ``limit`` clips nothing; with alpha = 1 and shift = 0
+    that is the gated SiLU form, W_down (silu(W_gate h) * W_up h)."""
 
     intermediate: int
-    limit: float
+    limit: float = float("inf")
     alpha: float = 1.702
+    shift: float = 1.0
+
+
+@dataclass(frozen=True)
+class ClippedGLUFFSpec:
+    """A dense feed-forward of the ``ClippedGLUSpec`` form.  ``names``: gate, up, down after the prefix."""
+
+    kind: ClassVar[str] = "clipped_glu"
+    hidden: int
+    glu: ClippedGLUSpec
+    names: tuple[str, str, str] = ("gate", "up", "down")
 
 
 @dataclass(frozen=True)
@@ -207,7 +249,11 @@ class MoESpec:
     """A mixture of ``experts`` clipped-GLU feed-forwards of which each token uses ``top``: router logits z = W_r h + b in
     32-bit, the ``top`` largest are chosen and weighted by the soft-max over the chosen logits alone; ``shared`` (or None)
     is one more expert that every token uses with weight 1.  Tensor names after the prefix: ``expert_prefix`` + index + "."
-    + gate / up / down, ``router`` and its bias, ``shared_prefix`` + gate / up / down."""
+    + gate / up / down, ``router`` and its bias ("" for none), ``shared_prefix`` + gate / up / down.
+    ``score`` = "sigmoid": the scores are s = sigmoid(z); the choice goes by s + correction (the tensor ``correction_name``
+    [experts], "" for none) and the weights are the chosen experts' s themselves, not renormalized.  ``groups`` > 1: the
+    experts form that many equal groups of neighbours; a group's score is the sum of its two largest choice scores, and only
+    experts of the ``keep_groups`` best groups can be chosen."""
 
     kind: ClassVar[str] = "moe"
     hidden: int
@@ -220,6 +266,10 @@ class MoESpec:
     router_name: str = "router"
     router_bias_name: str = "router.b"
     shared_prefix: str = "shared."
+    score: str = "softmax"
+    correction_name: str = ""
+    groups: int = 1
+    keep_groups: int = 1
 
 
 @dataclass(frozen=True)
@@ -322,10 +372,23 @@ class LayerCall:
     """One entry of the run order.  ``layer`` indexes ``ModelSpec.layers`` (a layer may be named
     by several entries: its weights are used again, each entry with a cache of its own).
     ``cache_from`` names an EARLIER entry of the run order whose cache this entry reads instead
-    of writing one of its own."""
+    of writing one of its own.  ``enters``: this entry is the first of pass number ``enters`` over a range of layers
+    (``ModelSpec.passes``): what the pass adds to the stream is added right before the entry runs."""
 
     layer: int
     cache_from: int | None = None
+    enters: int | None = None
+
+
+@dataclass(frozen=True)
+class PassSpec:
+    """What is added to the residual stream in front of each pass over a range of layers that runs several times with the
+    same weights: row t of the tensor ``name`` [times, hidden] in front of pass t, and, in front of every pass but the
+    first if ``add_embedding``, the embedding's output (the stream as it was before the first layer)."""
+
+    name: str
+    times: int
+    add_embedding: bool = True
 
 
 @dataclass(frozen=True)
@@ -363,11 +426,14 @@ class ModelSpec:
     # sublayer that a layer does not have); anything else that is unexpected is an error
     unread_prefixes: tuple[str, ...] = field(default_factory=tuple)
     pair_embedding: PairEmbeddingSpec | None = None  # models that carry 32-bit streams only
+    passes: PassSpec | None = None  # models that carry 32-bit streams only; see ``LayerCall.enters``
 
     def __post_init__(self) -> None:
         for pos, call in enumerate(self.run_order):
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"run order entry {pos} names layer {call.layer}, but there are {len(self.layers)} layers")
+            if call.enters is not None and (self.passes is None or not 0 <= call.enters < self.passes.times):
+                raise ValueError(f"run order entry {pos} starts pass {call.enters}, which the model does not have")
             if call.cache_from is not None:
                 if not 0 <= call.cache_from < pos:
                     raise ValueError(f"run order entry {pos} reads the cache of entry {call.cache_from}, which is not an earlier entry")

@@ -8,7 +8,7 @@
 // Options that the reference's attention does not have, each off at 0: ``chunk`` (a query also sees no key before the
 // start of its own chunk, floor(p / chunk) * chunk, chunks counted from position 0), ``cap`` (a score s, after the
 // scale, becomes cap * tanh(s / cap)), ``sink`` (the soft-max's denominator holds one more term of score 0 that has no
-// value), values of another size ``vd`` than the keys' ``hd``, and ``slope_exp`` (a bias by distance: head h of H loses
+// value; with ``sink_logit`` [heads] the term is exp(sink_logit[h]) instead, a learned number that is not scaled), values of another size ``vd`` than the keys' ``hd``, and ``slope_exp`` (a bias by distance: head h of H loses
 // 2^(-slope_exp (h + 1) / H) * (p - key) from its score, after the cap).
 // Query head h reads key/value head h / (heads / kv_heads).    (reference: model/attention.py:33)
 // K pages: [page][kv head][token][hd];  V pages: [page][kv head][vd][token].
@@ -23,7 +23,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     T* __restrict__ out, const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ token_req, const int* __restrict__ positions,
     const int* __restrict__ block_table, int table_stride, int heads, int kv_heads, int hd, int vd, int page_size, float scale,
-    int window, int chunk, float cap, int sink, float slope_exp) {
+    int window, int chunk, float cap, int sink, const float* __restrict__ sink_logit, float slope_exp) {
   extern __shared__ float smem[];  // q_s[hd] | p_s[AG_THREADS] | scratch[16]
   float* q_s = smem;
   float* p_s = smem + hd;
@@ -77,7 +77,10 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     }
     __syncthreads();
   }
-  if (sink) l += expf(-m);  // the term of score 0, in the units of the running maximum
+  if (sink_logit)
+    l += expf(sink_logit[h] - m);  // the learned term, in the units of the running maximum
+  else if (sink)
+    l += expf(-m);  // the term of score 0
 #pragma unroll
   for (int ci = 0; ci < AG_MAX_VD / AG_THREADS; ++ci)
     if (tid + ci * AG_THREADS < vd) out[((size_t)t * heads + h) * vd + tid + ci * AG_THREADS] = from_f<T>(acc[ci] / l);
@@ -86,7 +89,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
 extern "C" int ns_attn_generic(void* out, const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                const int* token_req, const int* positions, const int* block_table, int table_stride,
                                int n_tokens, int heads, int kv_heads, int hd, int vd, int page_size, float scale, int window,
-                               int chunk, float cap, int sink, float slope_exp, int dtype, hipStream_t stream) {
+                               int chunk, float cap, int sink, const float* sink_logit, float slope_exp, int dtype, hipStream_t stream) {
   if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || hd <= 0 || hd > 1024 || vd <= 0 || vd > AG_MAX_VD || page_size <= 0 ||
       window < 0 || chunk < 0 || cap < 0.f || slope_exp < 0.f)
     return NS_ERR_BAD_ARG;
@@ -95,10 +98,10 @@ extern "C" int ns_attn_generic(void* out, const void* q, int q_stride, const voi
   const size_t smem = (size_t)(hd + AG_THREADS + 16) * sizeof(float);
   if (dtype == NS_DTYPE_F32)
     attn_generic_kernel<float><<<grid, AG_THREADS, smem, stream>>>((float*)out, (const float*)q, q_stride, (const float*)k_cache,
-        (const float*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, vd, page_size, scale, window, chunk, cap, sink, slope_exp);
+        (const float*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, vd, page_size, scale, window, chunk, cap, sink, sink_logit, slope_exp);
   else if (dtype == NS_DTYPE_BF16)
     attn_generic_kernel<bf16_t><<<grid, AG_THREADS, smem, stream>>>((bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
-        (const bf16_t*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, vd, page_size, scale, window, chunk, cap, sink, slope_exp);
+        (const bf16_t*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, vd, page_size, scale, window, chunk, cap, sink, sink_logit, slope_exp);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();
@@ -173,6 +176,8 @@ extern "C" int ns_unit_kv_write(void* qkv, int stride, const int* positions, con
 //   q <- (q + bq) / sqrt(mean((q + bq)^2 over heads*hd) + eps) * qw         (in place)
 //   k <- likewise over kv_heads*hd with kw                                   (into the K pages)
 //   v <- v + bv;  v <- (1 - lambda) v + lambda v_other  if v_other is given   (into the V pages; also to v_keep if given)
+// With ``form.rot`` > 0 the first ``rot`` channels of every head of q and k are then rotated by the token's position
+// (``inv_freq`` [rot / 2]); a thread owns both channels of a pair.
 // ``bias`` [heads*hd + kv_heads*(hd + vd)], ``qw``, ``kw`` and ``lambda`` (one value) may each be null.  One workgroup a token.
 // ------------------------------------------------------------------------------------------------
 template <typename T>
@@ -180,7 +185,8 @@ __global__ __launch_bounds__(256) void whole_norm_kv_write_kernel(
     T* __restrict__ qkv, int stride, const T* __restrict__ bias, const T* __restrict__ qw, const T* __restrict__ kw,
     const T* __restrict__ lambda, const T* __restrict__ v_other, int v_other_stride, T* __restrict__ v_keep, int v_keep_stride,
     const int* __restrict__ positions, const int* __restrict__ token_req, const int* __restrict__ block_table, int table_stride,
-    T* __restrict__ k_cache, T* __restrict__ v_cache, int heads, int kv_heads, int hd, int vd, int page_size, float eps) {
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int heads, int kv_heads, int hd, int vd, int page_size, float eps,
+    const float* __restrict__ inv_freq, RopeForm form) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   T* row = qkv + (size_t)t * stride;
@@ -205,11 +211,40 @@ __global__ __launch_bounds__(256) void whole_norm_kv_write_kernel(
     }
     fk = 1.f / sqrtf(block_sum(ss, scratch) / (float)nk + eps);
   }
+  if (form.rot > 0) {
+    // the rotated pairs of q and of k: item = (head among q heads then k heads, pair)
+    const int half = form.rot / 2;
+    for (int i = threadIdx.x; i < (heads + kv_heads) * half; i += blockDim.x) {
+      const int h = i / half, j = i % half;
+      const bool is_q = h < heads;
+      int d1, d2;
+      rope_pair_channels(form, j, d1, d2);
+      const int at = h * hd;  // q heads and k heads follow each other in the row
+      const T* w = is_q ? qw : kw;
+      const int wat = is_q ? at : at - nq;
+      const float f = is_q ? fq : fk;
+      float a = to_f(row[at + d1]) + (bias ? to_f(bias[at + d1]) : 0.f), b = to_f(row[at + d2]) + (bias ? to_f(bias[at + d2]) : 0.f);
+      if (w) a = a * f * to_f(w[wat + d1]), b = b * f * to_f(w[wat + d2]);
+      float c, sn;
+      rope_cos_sin(form, pos, inv_freq[j], c, sn);
+      rope_turn(a, b, c, sn, a, b);
+      if (is_q) {
+        row[at + d1] = from_f<T>(a);
+        row[at + d2] = from_f<T>(b);
+      } else {
+        T* kd = k_cache + (((size_t)page * kv_heads + (h - heads)) * page_size + slot) * hd;
+        kd[d1] = from_f<T>(a);
+        kd[d2] = from_f<T>(b);
+      }
+    }
+  }
   for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+    if (i % hd < form.rot) continue;
     const float v = to_f(row[i]) + (bias ? to_f(bias[i]) : 0.f);
     row[i] = from_f<T>(qw ? v * fq * to_f(qw[i]) : v);
   }
   for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+    if (i % hd < form.rot) continue;
     const float v = to_f(row[nq + i]) + (bias ? to_f(bias[nq + i]) : 0.f);
     k_cache[(((size_t)page * kv_heads + i / hd) * page_size + slot) * hd + i % hd] = from_f<T>(kw ? v * fk * to_f(kw[i]) : v);
   }
@@ -226,17 +261,19 @@ __global__ __launch_bounds__(256) void whole_norm_kv_write_kernel(
 extern "C" int ns_whole_norm_kv_write(void* qkv, int stride, const void* bias, const void* qw, const void* kw, const void* lambda,
                                       const void* v_other, int v_other_stride, void* v_keep, int v_keep_stride, const int* positions,
                                       const int* token_req, const int* block_table, int table_stride, void* k_cache, void* v_cache,
-                                      int n_tokens, int heads, int kv_heads, int hd, int vd, int page_size, float eps, int dtype,
-                                      hipStream_t stream) {
+                                      int n_tokens, int heads, int kv_heads, int hd, int vd, int page_size, float eps, const float* inv_freq,
+                                      int rot, int interleaved, float factor, int dtype, hipStream_t stream) {
   if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || hd <= 0 || vd <= 0 || page_size <= 0) return NS_ERR_BAD_ARG;
+  if (rot < 0 || rot > hd || rot % 2 || (rot > 0 && !inv_freq)) return NS_ERR_BAD_ARG;
+  const RopeForm form{rot, interleaved, factor};
   if (dtype == NS_DTYPE_F32)
     whole_norm_kv_write_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, stride, (const float*)bias, (const float*)qw, (const float*)kw,
         (const float*)lambda, (const float*)v_other, v_other_stride, (float*)v_keep, v_keep_stride, positions, token_req, block_table,
-        table_stride, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, vd, page_size, eps);
+        table_stride, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, vd, page_size, eps, inv_freq, form);
   else if (dtype == NS_DTYPE_BF16)
     whole_norm_kv_write_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((bf16_t*)qkv, stride, (const bf16_t*)bias, (const bf16_t*)qw, (const bf16_t*)kw,
         (const bf16_t*)lambda, (const bf16_t*)v_other, v_other_stride, (bf16_t*)v_keep, v_keep_stride, positions, token_req, block_table,
-        table_stride, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, vd, page_size, eps);
+        table_stride, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, vd, page_size, eps, inv_freq, form);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();

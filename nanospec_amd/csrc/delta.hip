@@ -429,9 +429,9 @@ extern "C" int ns_delta_scan(float* o, const float* qkv, int C, const float* g, 
 // ------------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void gated_rms_kernel(T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ gate, int gate_stride,
-                                 const float* __restrict__ w, int w_stride, const float* __restrict__ den, int H, int E, float eps) {
+                                 const float* __restrict__ w, int w_stride, const float* __restrict__ den, int H, int E, float eps, int silu) {
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  w += (size_t)h * w_stride;  // 0: all heads share one weight
+  if (w) w += (size_t)h * w_stride;  // 0: all heads share one weight; no weight at all: the factor is 1
   const float* p = o + ((size_t)r * H + h) * E;
   const float dinv = den ? 1.f / den[(size_t)r * H + h] : 1.f;  // a head's read-out that comes undivided
   float ss = 0.f;
@@ -443,18 +443,19 @@ __global__ void gated_rms_kernel(T* __restrict__ out, const float* __restrict__ 
   const float rinv = 1.f / sqrtf(ss / (float)E + eps);
   for (int e = lane; e < E; e += NS_WAVE) {
     const float z = to_f(gate[(size_t)r * gate_stride + (size_t)h * E + e]);
-    out[((size_t)r * H + h) * E + e] = from_f<T>(p[e] * dinv * rinv * w[e] / (1.f + expf(-z)));
+    // the gate: sigmoid(z), or with ``silu`` z sigmoid(z)
+    out[((size_t)r * H + h) * E + e] = from_f<T>(p[e] * dinv * rinv * (w ? w[e] : 1.f) * (silu ? z : 1.f) / (1.f + expf(-z)));
   }
 }
 
 extern "C" int ns_gated_rms(void* out, const float* o, const void* gate, int gate_stride, const float* w, int w_stride, const float* den,
-                            int n_tokens, int H, int E, float eps, int dtype, hipStream_t stream) {
+                            int n_tokens, int H, int E, float eps, int silu, int dtype, hipStream_t stream) {
   if (n_tokens <= 0 || H <= 0 || H > 65535 || E <= 0) return NS_ERR_BAD_ARG;
   dim3 grid(n_tokens, H);
   if (dtype == NS_DTYPE_F32)
-    gated_rms_kernel<float><<<grid, NS_WAVE, 0, stream>>>((float*)out, o, (const float*)gate, gate_stride, w, w_stride, den, H, E, eps);
+    gated_rms_kernel<float><<<grid, NS_WAVE, 0, stream>>>((float*)out, o, (const float*)gate, gate_stride, w, w_stride, den, H, E, eps, silu);
   else if (dtype == NS_DTYPE_BF16)
-    gated_rms_kernel<bf16_t><<<grid, NS_WAVE, 0, stream>>>((bf16_t*)out, o, (const bf16_t*)gate, gate_stride, w, w_stride, den, H, E, eps);
+    gated_rms_kernel<bf16_t><<<grid, NS_WAVE, 0, stream>>>((bf16_t*)out, o, (const bf16_t*)gate, gate_stride, w, w_stride, den, H, E, eps, silu);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();

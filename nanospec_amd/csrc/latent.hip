@@ -5,7 +5,7 @@
 // so the attention itself runs over ONE key/value head whose key is [c | r] (C + R channels) and whose value is c, with
 // queries [Uk_h^T q_h | qr_h]; the kernels here are what surrounds it:
 //   latent_prep      the row [dq | dkv | gate] of the first product -> normed query latent, [c | r] into the K page,
-//                    c into the V page, sigmoid of the gate logits (32-bit)
+//                    c into the V page, sigmoid of the gate logits (32-bit); a layer without a query latent has no dq part
 //   latent_q_absorb  q [H][D + R] -> [H][C + R]: the unrotated part through Uk_h^T, the rotated part turned by its position
 //   latent_out       o [H][C] -> [H][E] through Uv_h, times the gate
 //   headwise_mfma    the two per-head products on the matrix cores (bfloat16, sizes that are multiples of 32 and 16)
@@ -28,7 +28,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
   const int slot = pos % page_size;
   float ss = 0.f;
   for (int i = threadIdx.x; i < q_rank; i += blockDim.x) ss = fmaf(to_f(row[i]), to_f(row[i]), ss);
-  const float fq = 1.f / sqrtf(block_sum(ss, scratch) / (float)q_rank + eps);
+  const float fq = q_rank > 0 ? 1.f / sqrtf(block_sum(ss, scratch) / (float)q_rank + eps) : 1.f;  // (no query latent: q_rank = 0)
   ss = 0.f;
   for (int i = threadIdx.x; i < C; i += blockDim.x) ss = fmaf(to_f(row[q_rank + i]), to_f(row[q_rank + i]), ss);
   const float fc = 1.f / sqrtf(block_sum(ss, scratch) / (float)C + eps);
@@ -56,7 +56,7 @@ extern "C" int ns_latent_prep(const void* proj, int stride, const void* qn_w, co
                               float* gate, const int* positions, const int* token_req, const int* block_table, int table_stride,
                               void* k_cache, void* v_cache, int n_tokens, int q_rank, int C, int R, int H, int page_size, float eps,
                               int dtype, hipStream_t stream) {
-  if (n_tokens <= 0 || q_rank <= 0 || C <= 0 || R < 0 || R % 2 || H < 0 || (H > 0 && !gate) || page_size <= 0) return NS_ERR_BAD_ARG;
+  if (n_tokens <= 0 || q_rank < 0 || (q_rank > 0 && (!cq || !qn_w)) || C <= 0 || R < 0 || R % 2 || H < 0 || (H > 0 && !gate) || page_size <= 0) return NS_ERR_BAD_ARG;
   if (dtype == NS_DTYPE_F32)
     latent_prep_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)proj, stride, (const float*)qn_w, (const float*)cn_w, inv_freq, factor,
         (float*)cq, gate, positions, token_req, block_table, table_stride, (float*)k_cache, (float*)v_cache, q_rank, C, R, H, page_size, eps);

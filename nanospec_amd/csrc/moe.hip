@@ -1,8 +1,10 @@
 // A mixture of small gated feed-forward experts, and the per-layer token input of a decoder that has one.
 //
 // Router: z = W_r h + b in 32-bit; the ``top`` largest logits are chosen (the lower index wins a tie) and weighted by the
-// soft-max over the chosen logits alone.
-// Expert (``clipped GLU``): g = min(W_gate h, limit); u = clamp(W_up h, -limit, limit); y = W_down (g sigmoid(alpha g) (u + 1)).
+// soft-max over the chosen logits alone; or sigmoid scores with a correction on the choice and groups of experts (see
+// ``moe_choose_kernel``).
+// Expert (``clipped GLU``): g = min(W_gate h, limit); u = clamp(W_up h, -limit, limit); y = W_down (g sigmoid(alpha g) (u + shift));
+// an infinite limit clips nothing, and with alpha = 1 and shift = 0 the expert is W_down (silu(W_gate h) * W_up h).
 // The experts' matrices are stacked: gate and up [experts][ff][W], down [experts][W][ff].
 #include "common.h"
 
@@ -50,20 +52,71 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(const T* __restrict__ h
   }
 }
 
-// A wave a token: the logits in LDS, every lane looks through its share for the largest one not yet taken, the lanes'
+// A wave a token: the choice scores in LDS, every lane looks through its share for the largest one not yet taken, the lanes'
 // candidates meet by lane exchange (the larger value wins, the lower index among equals; what is no number counts as
 // minus infinity, so a row of anything still chooses ``top`` different experts).
+// ``sigmoid`` = 0: the choice goes by the logits and the weights are the soft-max over the chosen logits.
+// ``sigmoid`` = 1: scores s = sigmoid(z); the choice goes by s + correction[e] (``correction`` may be null) and the weights are
+// the chosen experts' s, not renormalized.  ``groups`` > 1: the experts form that many equal groups of neighbours; a group's
+// score is the sum of its two largest choice scores (of its one, if it has one), and only the ``keep`` best groups' experts
+// can be chosen: the others never enter the comparison, whatever their scores' sign.
+__device__ __forceinline__ void wave_best(float& bv, int& best) {
+#pragma unroll
+  for (int o = NS_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, NS_WAVE);
+    const int oi = __shfl_xor(best, o, NS_WAVE);
+    if (oi >= 0 && (best < 0 || ov > bv || (ov == bv && oi < best))) best = oi, bv = ov;
+  }
+}
+
 __global__ __launch_bounds__(64) void moe_choose_kernel(const float* __restrict__ z, int* __restrict__ sel, float* __restrict__ wt, int n,
-                                                        int experts, int top) {
-  __shared__ float zs[MOE_MAX_EXPERTS];
+                                                        int experts, int top, int sigmoid, const float* __restrict__ correction, int groups,
+                                                        int keep) {
+  __shared__ float zs[MOE_MAX_EXPERTS];   // choice scores
+  __shared__ float ws[MOE_MAX_EXPERTS];   // what the weights are made from: the logits, or the sigmoid scores
+  __shared__ float gs[MOE_MAX_EXPERTS];   // group scores
   __shared__ unsigned char taken[MOE_MAX_EXPERTS];
+  __shared__ unsigned char gkept[MOE_MAX_EXPERTS];
   const int t = blockIdx.x, lane = threadIdx.x;
   for (int e = lane; e < experts; e += NS_WAVE) {
-    const float v = z[(size_t)t * experts + e];
+    float v = z[(size_t)t * experts + e];
+    if (sigmoid) {
+      v = 1.f / (1.f + expf(-v));
+      ws[e] = v;
+      if (correction) v += correction[e];
+    } else {
+      ws[e] = v;
+    }
     zs[e] = v == v ? v : -INFINITY;
     taken[e] = 0;
   }
   __syncthreads();
+  if (groups > 1) {
+    const int per = experts / groups;
+    for (int g = lane; g < groups; g += NS_WAVE) {
+      float a = -INFINITY, b = -INFINITY;  // the two largest of the group
+      for (int e = g * per; e < (g + 1) * per; ++e) {
+        const float v = zs[e];
+        if (v > a) b = a, a = v;
+        else if (v > b) b = v;
+      }
+      gs[g] = per > 1 ? a + b : a;
+      gkept[g] = 0;
+    }
+    __syncthreads();
+    for (int k = 0; k < keep; ++k) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int g = lane; g < groups; g += NS_WAVE)
+        if (!gkept[g] && (best < 0 || gs[g] > bv)) best = g, bv = gs[g];
+      wave_best(bv, best);
+      if (lane == 0) gkept[best] = 1;
+      __syncthreads();
+    }
+    for (int e = lane; e < experts; e += NS_WAVE)
+      if (!gkept[e / per]) taken[e] = 1;
+    __syncthreads();
+  }
   float largest = 0.f, sum = 0.f, mine = 0.f;  // lane k keeps the k-th chosen value
   int mine_idx = 0;
   for (int k = 0; k < top; ++k) {
@@ -71,29 +124,30 @@ __global__ __launch_bounds__(64) void moe_choose_kernel(const float* __restrict_
     float bv = -INFINITY;
     for (int e = lane; e < experts; e += NS_WAVE)
       if (!taken[e] && (best < 0 || zs[e] > bv)) best = e, bv = zs[e];
-#pragma unroll
-    for (int o = NS_WAVE / 2; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(bv, o, NS_WAVE);
-      const int oi = __shfl_xor(best, o, NS_WAVE);
-      if (oi >= 0 && (best < 0 || ov > bv || (ov == bv && oi < best))) best = oi, bv = ov;
-    }
+    wave_best(bv, best);
     if (lane == 0) taken[best] = 1;
-    if (k == 0) largest = bv;
-    const float w = expf(bv - largest);
+    float w;
+    if (sigmoid) {
+      w = ws[best];
+    } else {
+      if (k == 0) largest = bv;
+      w = expf(bv - largest);
+    }
     sum += w;
     if (lane == k % NS_WAVE && k < NS_WAVE) mine = w, mine_idx = best;
     __syncthreads();
   }
   if (lane < top) {
     sel[(size_t)t * top + lane] = mine_idx;
-    wt[(size_t)t * top + lane] = mine / sum;
+    wt[(size_t)t * top + lane] = sigmoid ? mine : mine / sum;
   }
 }
 
 // ``z``: scratch, float32 [n][experts]
 extern "C" int ns_moe_route(const void* h, int h_stride, const float* wr, const float* br, float* z, int* sel, float* wt, int n, int W, int experts,
-                            int top, int dtype, hipStream_t stream) {
+                            int top, int sigmoid, const float* correction, int groups, int keep, int dtype, hipStream_t stream) {
   if (n <= 0 || W <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > MOE_MAX_TOP || top > experts) return NS_ERR_BAD_ARG;
+  if (groups < 1 || experts % groups || keep < 1 || keep > groups || top > keep * (experts / groups)) return NS_ERR_BAD_ARG;
   dim3 grid((n + ROUTE_TOK - 1) / ROUTE_TOK, (experts + 3) / 4);
   if (grid.y > 65535) return NS_ERR_UNSUPPORTED;
   const size_t elem = dtype == NS_DTYPE_F32 ? 4 : 2;
@@ -104,14 +158,14 @@ extern "C" int ns_moe_route(const void* h, int h_stride, const float* wr, const 
     moe_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)h, h_stride, wr, br, z, n, W, experts, vec);
   else
     return NS_ERR_UNSUPPORTED;
-  moe_choose_kernel<<<n, 64, 0, stream>>>(z, sel, wt, n, experts, top);
+  moe_choose_kernel<<<n, 64, 0, stream>>>(z, sel, wt, n, experts, top, sigmoid, correction, groups, keep);
   return ns_launch_status();
 }
 
-__device__ __forceinline__ float clipped_glu(float g, float u, float limit, float alpha) {
+__device__ __forceinline__ float clipped_glu(float g, float u, float limit, float alpha, float shift) {
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
-  return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+  return g / (1.f + expf(-alpha * g)) * (u + shift);
 }
 
 // ------------------------------------------------------------------------------------------------ few rows
@@ -159,7 +213,7 @@ __device__ __forceinline__ float row_dot(const T* __restrict__ w, const float* _
 template <typename T>
 __global__ __launch_bounds__(256) void moe_rows_up_kernel(const T* __restrict__ h, int h_stride, const T* __restrict__ wg, const T* __restrict__ wu,
                                                           const int* __restrict__ sel, float* __restrict__ act, int W, int ff, int top, int per,
-                                                          float limit, float alpha, int vec) {
+                                                          float limit, float alpha, float shift, int vec) {
   extern __shared__ __attribute__((aligned(16))) float moe_lds[];  // [W]
   const int t = blockIdx.z, k = blockIdx.y, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE, waves = blockDim.x / NS_WAVE;
   const int e = sel[(size_t)t * top + k];
@@ -169,7 +223,7 @@ __global__ __launch_bounds__(256) void moe_rows_up_kernel(const T* __restrict__ 
   for (int f = f0 + wave; f < f1; f += waves) {
     const size_t row = ((size_t)e * ff + f) * W;
     const float g = row_dot(wg + row, moe_lds, W, lane, vec), u = row_dot(wu + row, moe_lds, W, lane, vec);
-    if (lane == 0) act[((size_t)t * top + k) * ff + f] = round_to<T>(clipped_glu(round_to<T>(g), round_to<T>(u), limit, alpha));
+    if (lane == 0) act[((size_t)t * top + k) * ff + f] = round_to<T>(clipped_glu(round_to<T>(g), round_to<T>(u), limit, alpha, shift));
   }
 }
 
@@ -198,7 +252,7 @@ static int moe_slice(int channels, int rows) {
 }
 
 extern "C" int ns_moe_expert_rows(const void* h, int h_stride, const void* wg, const void* wu, const void* wd, const int* sel, const float* wt,
-                                  float* act, float* out, int n, int W, int ff, int top, float limit, float alpha, int dtype, hipStream_t stream) {
+                                  float* act, float* out, int n, int W, int ff, int top, float limit, float alpha, float shift, int dtype, hipStream_t stream) {
   if (n <= 0 || n > 65535 || W <= 0 || ff <= 0 || top <= 0 || top > 65535) return NS_ERR_BAD_ARG;
   if ((size_t)W * sizeof(float) > 64 * 1024 || (size_t)ff * sizeof(float) > 64 * 1024) return NS_ERR_UNSUPPORTED;
   const size_t elem = dtype == NS_DTYPE_F32 ? 4 : 2;
@@ -208,11 +262,11 @@ extern "C" int ns_moe_expert_rows(const void* h, int h_stride, const void* wg, c
   dim3 g1((ff + per_f - 1) / per_f, top, n), g2((W + per_c - 1) / per_c, top, n);
   if (dtype == NS_DTYPE_F32) {
     moe_rows_up_kernel<float><<<g1, 256, W * sizeof(float), stream>>>((const float*)h, h_stride, (const float*)wg, (const float*)wu, sel, act, W, ff,
-                                                                       top, per_f, limit, alpha, vec_up);
+                                                                       top, per_f, limit, alpha, shift, vec_up);
     moe_rows_down_kernel<float><<<g2, 256, ff * sizeof(float), stream>>>(act, (const float*)wd, sel, wt, out, W, ff, top, per_c, vec_down);
   } else if (dtype == NS_DTYPE_BF16) {
     moe_rows_up_kernel<bf16_t><<<g1, 256, W * sizeof(float), stream>>>((const bf16_t*)h, h_stride, (const bf16_t*)wg, (const bf16_t*)wu, sel, act, W,
-                                                                        ff, top, per_f, limit, alpha, vec_up);
+                                                                        ff, top, per_f, limit, alpha, shift, vec_up);
     moe_rows_down_kernel<bf16_t><<<g2, 256, ff * sizeof(float), stream>>>(act, (const bf16_t*)wd, sel, wt, out, W, ff, top, per_c, vec_down);
   } else {
     return NS_ERR_UNSUPPORTED;
@@ -271,7 +325,7 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16_t* __restrict
                                                         const bf16_t* __restrict__ B1, const int* __restrict__ perm,
                                                         const int* __restrict__ tile_e, const int* __restrict__ tile_r0,
                                                         const int* __restrict__ tile_rows, bf16_t* __restrict__ act_out, float* __restrict__ out,
-                                                        const float* __restrict__ wt, int N, int K, int top, float limit, float alpha) {
+                                                        const float* __restrict__ wt, int N, int K, int top, float limit, float alpha, float shift) {
   __shared__ __attribute__((aligned(16))) bf16_t As[MG_TM * MG_LD];
   __shared__ __attribute__((aligned(16))) bf16_t Bs[(DUAL ? 2 : 1) * MG_TN * MG_LD];
   const int tile = blockIdx.y, e = tile_e[tile];
@@ -370,7 +424,7 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16_t* __restrict
         const int col = n0 + MG_TN / 2 * wn + 16 * j + r;
         if (col >= N) continue;
         if (DUAL)
-          act_out[(size_t)slot * N + col] = from_f<bf16_t>(clipped_glu(round_to<bf16_t>(acc0[i][j][q]), round_to<bf16_t>(acc1[i][j][q]), limit, alpha));
+          act_out[(size_t)slot * N + col] = from_f<bf16_t>(clipped_glu(round_to<bf16_t>(acc0[i][j][q]), round_to<bf16_t>(acc1[i][j][q]), limit, alpha, shift));
         else
           out[(size_t)pair * N + col] = share * acc0[i][j][q];
       }
@@ -382,7 +436,7 @@ extern "C" int ns_moe_group_tiles(int pairs, int experts) { return (pairs + MG_T
 
 // ``ints``: scratch of pairs + 3 * ns_moe_group_tiles(pairs, experts) 32-bit words; ``act``: bfloat16 [pairs][ff]
 extern "C" int ns_moe_expert_groups(const void* h, int h_stride, const void* wg, const void* wu, const void* wd, const int* sel, const float* wt,
-                                    int* ints, void* act, float* out, int n, int W, int ff, int top, int experts, float limit, float alpha,
+                                    int* ints, void* act, float* out, int n, int W, int ff, int top, int experts, float limit, float alpha, float shift,
                                     hipStream_t stream) {
   if (n <= 0 || W <= 0 || ff <= 0 || top <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS) return NS_ERR_BAD_ARG;
   if (W % 8 || ff % 8 || h_stride % 8 || (uintptr_t)h % 16 || (uintptr_t)wg % 16 || (uintptr_t)wu % 16 || (uintptr_t)wd % 16 || (uintptr_t)act % 16)
@@ -398,30 +452,30 @@ extern "C" int ns_moe_expert_groups(const void* h, int h_stride, const void* wg,
   if (tiles > 65535) return NS_ERR_UNSUPPORTED;
   dim3 g1((ff + MG_TN - 1) / MG_TN, tiles), g2((W + MG_TN - 1) / MG_TN, tiles);
   moe_group_kernel<true><<<g1, 256, 0, stream>>>((const bf16_t*)h, h_stride, (const bf16_t*)wg, (const bf16_t*)wu, perm, tile_e, tile_r0, tile_rows,
-                                                  (bf16_t*)act, nullptr, nullptr, ff, W, top, limit, alpha);
+                                                  (bf16_t*)act, nullptr, nullptr, ff, W, top, limit, alpha, shift);
   moe_group_kernel<false><<<g2, 256, 0, stream>>>((const bf16_t*)act, ff, (const bf16_t*)wd, nullptr, perm, tile_e, tile_r0, tile_rows, nullptr, out,
-                                                   wt, W, ff, top, limit, alpha);
+                                                   wt, W, ff, top, limit, alpha, shift);
   return ns_launch_status();
 }
 
 // out[t][f] = clipped_glu(gu[t][f], gu[t][ff + f]) for the result of a product with the stacked [gate; up] matrix
 template <typename T>
-__global__ void clipped_glu_kernel(T* __restrict__ out, const T* __restrict__ gu, int gu_stride, int ff, size_t count, float limit, float alpha) {
+__global__ void clipped_glu_kernel(T* __restrict__ out, const T* __restrict__ gu, int gu_stride, int ff, size_t count, float limit, float alpha, float shift) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
     const size_t t = i / ff, f = i % ff;
-    out[i] = from_f<T>(clipped_glu(to_f(gu[t * gu_stride + f]), to_f(gu[t * gu_stride + ff + f]), limit, alpha));
+    out[i] = from_f<T>(clipped_glu(to_f(gu[t * gu_stride + f]), to_f(gu[t * gu_stride + ff + f]), limit, alpha, shift));
   }
 }
 
-extern "C" int ns_clipped_glu(void* out, const void* gu, int gu_stride, int n, int ff, float limit, float alpha, int dtype, hipStream_t stream) {
+extern "C" int ns_clipped_glu(void* out, const void* gu, int gu_stride, int n, int ff, float limit, float alpha, float shift, int dtype, hipStream_t stream) {
   if (n <= 0 || ff <= 0) return NS_ERR_BAD_ARG;
   const size_t count = (size_t)n * ff;
   size_t blocks = (count + 255) / 256;
   if (blocks > 65535) blocks = 65535;
   if (dtype == NS_DTYPE_F32)
-    clipped_glu_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)out, (const float*)gu, gu_stride, ff, count, limit, alpha);
+    clipped_glu_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)out, (const float*)gu, gu_stride, ff, count, limit, alpha, shift);
   else if (dtype == NS_DTYPE_BF16)
-    clipped_glu_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, gu_stride, ff, count, limit, alpha);
+    clipped_glu_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, gu_stride, ff, count, limit, alpha, shift);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();

@@ -417,3 +417,37 @@ extern "C" int ns_activation(void* out, const void* x, size_t count, int act, in
     activation_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, count, act);
   return ns_launch_status();
 }
+
+// What a pass over a range of layers that runs several times adds to the streams in front of it:
+//   x[r][s][:] += scale * table[ids[r]][:]  (the embedding's output again, if ``table``)  +  vec[:]  (if ``vec``)
+// for every copy s, in 32-bit.  ``table`` and ``vec`` are in the model's storage type.
+template <typename T>
+__global__ void stream_add_rows_kernel(float* __restrict__ x, const T* __restrict__ table, const int* __restrict__ ids, const T* __restrict__ vec,
+                                       int hidden, int copies, float scale) {
+  const int row = blockIdx.x;
+  const T* src = table ? table + (size_t)ids[row] * hidden : nullptr;
+  float* dst = x + (size_t)row * copies * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    // (the two terms are added to the stream one after the other, as they are defined)
+    const float e = src ? to_f(src[i]) * scale : 0.f, v = vec ? to_f(vec[i]) : 0.f;
+    for (int s = 0; s < copies; ++s) {
+      float cur = dst[(size_t)s * hidden + i];
+      if (src) cur += e;
+      if (vec) cur += v;
+      dst[(size_t)s * hidden + i] = cur;
+    }
+  }
+}
+
+extern "C" int ns_stream_add_rows(float* x, const void* table, const int* ids, const void* vec, int n_tokens, int hidden, int copies, float scale,
+                                  int dtype, hipStream_t stream) {
+  if (n_tokens <= 0 || hidden <= 0 || copies <= 0 || copies > NS_MAX_STREAMS || (table && !ids)) return NS_ERR_BAD_ARG;
+  if (!table && !vec) return NS_OK;
+  if (dtype == NS_DTYPE_F32)
+    stream_add_rows_kernel<float><<<n_tokens, 256, 0, stream>>>(x, (const float*)table, ids, (const float*)vec, hidden, copies, scale);
+  else if (dtype == NS_DTYPE_BF16)
+    stream_add_rows_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(x, (const bf16_t*)table, ids, (const bf16_t*)vec, hidden, copies, scale);
+  else
+    return NS_ERR_UNSUPPORTED;
+  return ns_launch_status();
+}

@@ -674,13 +674,16 @@ def _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim, v_dim: int 
 
 def attention_generic(q, out, k_cache, v_cache, token_req, positions, block_table, heads: int, kv_heads: int, head_dim: int,
                       scale: float, window: int = 0, v_dim: int | None = None, chunk: int = 0, cap: float = 0.0,
-                      sink: bool = False, slope_exp: float = 0.0) -> torch.Tensor:
+                      sink: bool = False, slope_exp: float = 0.0, sink_logits: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of every token's query over its request's pages; any key and value size up to 1024, either
     dtype.  ``chunk`` > 0: a query sees no key before the start of its own chunk of positions; ``cap`` > 0: scores become
     cap * tanh(score / cap); ``sink``: one more term of score 0 without a value in the soft-max's denominator;
-    ``slope_exp`` > 0: head h of H loses 2^(-slope_exp (h + 1) / H) times its distance to the key from every score."""
+    ``slope_exp`` > 0: head h of H loses 2^(-slope_exp (h + 1) / H) times its distance to the key from every score.
+    ``sink_logits`` (float32 [heads]): the one more term is exp(sink_logits[h]), not scaled, instead of exp(0)."""
     v_dim = head_dim if v_dim is None else v_dim
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim, v_dim)
+    if sink_logits is not None and (_f32(sink_logits, "sink_logits").numel() != heads):
+        raise KernelRefused(f"attention_generic: sink_logits holds one float32 value for each of the {heads} heads")
     _i32(token_req, "token_req"), _i32(positions, "positions"), _i32(block_table, "block_table")
     if head_dim > 1024 or v_dim > 1024:
         raise KernelRefused(f"attention_generic takes key and value sizes up to 1024, not {head_dim} and {v_dim}")
@@ -688,8 +691,8 @@ def attention_generic(q, out, k_cache, v_cache, token_req, positions, block_tabl
     _check(build.core().ns_attn_generic(_ptr(out), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(token_req),
                                         _ptr(positions), _ptr(block_table), c_int(block_table.stride(0)), c_int(n), c_int(heads),
                                         c_int(kv_heads), c_int(head_dim), c_int(v_dim), c_int(page), c_float(scale), c_int(window),
-                                        c_int(chunk), c_float(cap), c_int(1 if sink else 0), c_float(slope_exp), c_int(_dtype_code(q)), _stream()),
-           "attention_generic")
+                                        c_int(chunk), c_float(cap), c_int(1 if sink else 0), _ptr(sink_logits), c_float(slope_exp), c_int(_dtype_code(q)),
+                                        _stream()), "attention_generic")
     return out
 
 
@@ -973,6 +976,22 @@ def stream_step(x: torch.Tensor, pending: "PendingWrite | None", coeff: torch.Te
     return out
 
 
+def stream_add_rows(x: torch.Tensor, table: torch.Tensor | None, ids: torch.Tensor | None, vec: torch.Tensor | None, scale: float = 1.0) -> None:
+    """In place, for every copy s of a 32-bit stream ``x`` [tokens, copies, hidden]: x[r, s] += scale * table[ids[r]] (if
+    ``table``) + vec (if ``vec`` [hidden]); ``table`` and ``vec`` in one storage type."""
+    _f32(x, "x")
+    _gpu(table, ids, vec)
+    if table is None and vec is None:
+        return
+    n, S, W = x.shape
+    any_t = table if table is not None else vec
+    if ((table is not None and (table.dim() != 2 or table.shape[1] != W or not table.is_contiguous() or ids is None or _i32(ids, "ids").numel() != n))
+            or (vec is not None and (vec.shape != (W,) or not vec.is_contiguous() or vec.dtype != any_t.dtype)) or S > MAX_STREAMS):
+        raise KernelRefused(f"stream_add_rows: table [rows, {W}] with ids [{n}], vec [{W}], of one dtype")
+    _check(build.core().ns_stream_add_rows(_ptr(x), _ptr(table), _ptr(ids), _ptr(vec), c_int(n), c_int(W), c_int(S), c_float(scale),
+                                           c_int(_dtype_code(any_t)), _stream()), "stream_add_rows")
+
+
 def embed_pair_streams(table: torch.Tensor, pair_table: torch.Tensor, ids, positions, token_req, qo_indptr, state_slots, last_token: torch.Tensor,
                        out: torch.Tensor, scale: float, buckets: int, mul_prev: int, mul_cur: int) -> torch.Tensor:
     """``embed_streams`` plus a row of a second table chosen by the token and the one before it in its sequence:
@@ -999,13 +1018,18 @@ def embed_pair_streams(table: torch.Tensor, pair_table: torch.Tensor, ids, posit
 def whole_norm_kv_write(qkv: torch.Tensor, positions, token_req, block_table, k_cache, v_cache, heads: int, kv_heads: int, head_dim: int,
                         v_dim: int, eps: float, bias: torch.Tensor | None = None, q_weight: torch.Tensor | None = None,
                         k_weight: torch.Tensor | None = None, mix: torch.Tensor | None = None, v_other: torch.Tensor | None = None,
-                        v_keep: torch.Tensor | None = None) -> None:
+                        v_keep: torch.Tensor | None = None, inv_freq: torch.Tensor | None = None, rotary_dim: int = 0, interleaved: bool = False,
+                        factor: float = 1.0) -> None:
     """For attention without rotation whose projections carry biases and whose queries and keys pass an RMS norm over the whole
     projection.  A row of ``qkv`` is q [heads * head_dim], k [kv_heads * head_dim], v [kv_heads * v_dim]; ``bias`` of that
     width is added; q (in place) and k become x / sqrt(mean(x^2 over the whole projection) + eps) * weight; v becomes
     (1 - mix) v + mix v_other where ``v_other`` [tokens, kv_heads * v_dim] is given (``mix``: one value on the device), is
-    copied to ``v_keep`` where that is given, and k and v go into the pages of their positions."""
-    _gpu(qkv, positions, token_req, block_table, k_cache, v_cache, bias, q_weight, k_weight, mix, v_other, v_keep)
+    copied to ``v_keep`` where that is given, and k and v go into the pages of their positions.  ``rotary_dim`` > 0: the first
+    so many channels of every head of q and k are rotated by the token's position after the norm (``inv_freq`` float32
+    [rotary_dim / 2]; pairing and ``factor`` as in ``rope_kv_write``)."""
+    _gpu(qkv, positions, token_req, block_table, k_cache, v_cache, bias, q_weight, k_weight, mix, v_other, v_keep, inv_freq)
+    if rotary_dim and (rotary_dim % 2 or rotary_dim > head_dim or inv_freq is None or _f32(inv_freq, "inv_freq").numel() < rotary_dim // 2):
+        raise KernelRefused("whole_norm_kv_write: the rotated part is an even number of a head's channels, with a frequency per pair")
     n = positions.numel()
     nq, nk, nv = heads * head_dim, kv_heads * head_dim, kv_heads * v_dim
     if qkv.dim() != 2 or qkv.shape[0] != n or qkv.shape[1] < nq + nk + nv or qkv.stride(1) != 1:
@@ -1030,7 +1054,8 @@ def whole_norm_kv_write(qkv: torch.Tensor, positions, token_req, block_table, k_
                                                c_int(v_keep.stride(0) if v_keep is not None else 0), _ptr(positions), _ptr(token_req),
                                                _ptr(block_table), c_int(block_table.stride(0)), _ptr(k_cache), _ptr(v_cache), c_int(n),
                                                c_int(heads), c_int(kv_heads), c_int(head_dim), c_int(v_dim), c_int(page), c_float(eps),
-                                               c_int(_dtype_code(qkv)), _stream()), "whole_norm_kv_write")
+                                               _ptr(inv_freq if rotary_dim else None), c_int(rotary_dim), c_int(1 if interleaved else 0),
+                                               c_float(factor), c_int(_dtype_code(qkv)), _stream()), "whole_norm_kv_write")
 
 
 def head_norm_rope_kv_write(qkv: torch.Tensor, positions, token_req, block_table, inv_freq, k_cache, v_cache, heads: int, kv_heads: int,
@@ -1128,12 +1153,76 @@ def memory_scan(proj: torch.Tensor, offsets: tuple[int, int, int, int, int], gat
 # ------------------------------------------------------------------------------------------------ mixture of experts
 
 
+def retention_prep(proj: torch.Tensor, offsets: tuple[int, int, int], positions, inv_freq: torch.Tensor | None, heads: int, key_dim: int,
+                   value_dim: int, rotary_dim: int, key_scale: float, out: torch.Tensor, interleaved: bool = False, factor: float = 1.0) -> torch.Tensor:
+    """Rows [.. q .. k .. v ..] of a stacked product (``offsets``: the columns where q, k and v start) -> ``out`` float32
+    [tokens, heads * (2 key_dim + value_dim)] = [q | k | v]: the first ``rotary_dim`` channels of every head of q and k rotated
+    by the token's position in 32-bit, k then multiplied by ``key_scale``."""
+    _gpu(proj, positions, inv_freq, out)
+    _i32(positions, "positions"), _f32(out, "out")
+    n = positions.numel()
+    q_off, k_off, v_off = offsets
+    row = heads * (2 * key_dim + value_dim)
+    need = max(q_off + heads * key_dim, k_off + heads * key_dim, v_off + heads * value_dim)
+    if (proj.dim() != 2 or proj.shape[0] != n or proj.shape[1] < need or proj.stride(1) != 1 or out.shape != (n, row) or not out.is_contiguous()
+            or rotary_dim % 2 or not 0 <= rotary_dim <= key_dim or (rotary_dim and (inv_freq is None or _f32(inv_freq, "inv_freq").numel() < rotary_dim // 2))):
+        raise KernelRefused(f"retention_prep: rows of at least {need} columns, out float32 [{n}, {row}], an even rotated part of a head")
+    _check(build.core().ns_retention_prep(_ptr(proj), c_int(proj.stride(0)), c_int(q_off), c_int(k_off), c_int(v_off), _ptr(positions),
+                                          _ptr(inv_freq if rotary_dim else None), _ptr(out), c_int(n), c_int(heads), c_int(key_dim), c_int(value_dim),
+                                          c_int(rotary_dim), c_int(1 if interleaved else 0), c_float(factor), c_float(key_scale),
+                                          c_int(_dtype_code(proj)), _stream()), "retention_prep")
+    return out
+
+
+RETENTION_MAX_KEY_DIM = 512  # key channels of a head that ``retention_scan`` takes (a column's channels are 8 to a lane of one wave)
+
+
+def retention_scan(qkv: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, qo_indptr, state_slots, heads: int, key_dim: int, value_dim: int,
+                   out: torch.Tensor) -> torch.Tensor:
+    """S <- decay_h S + k v^T and out = S^T q per head over every request's tokens of the step in order.  ``qkv`` float32
+    [tokens, heads * (2 key_dim + value_dim)] as ``retention_prep`` leaves it; ``decay`` float32 [heads]; ``state`` float32
+    [slots, >= heads * value_dim * key_dim], a request's S as [heads, value_dim, key_dim] in its slot; ``out`` float32 [tokens,
+    heads * value_dim]."""
+    _f32(qkv, "qkv"), _f32(decay, "decay"), _f32(out, "out"), _i32(qo_indptr, "qo_indptr"), _i32(state_slots, "state_slots")
+    if state.dtype != torch.float32 or state.dim() != 2 or not state.is_contiguous() or not state.is_cuda:
+        raise KernelRefused("retention_scan: the state is float32 [slots, floats per slot] on the GPU")
+    stride = state.shape[1]
+    n = qkv.shape[0]
+    if (key_dim > RETENTION_MAX_KEY_DIM or qkv.shape != (n, heads * (2 * key_dim + value_dim)) or decay.numel() != heads or out.shape != (n, heads * value_dim)
+            or stride < heads * key_dim * value_dim or qo_indptr.numel() != state_slots.numel() + 1):
+        raise KernelRefused(f"retention_scan: operands do not fit {heads} heads of {key_dim} x {value_dim} (key sizes up to {RETENTION_MAX_KEY_DIM})")
+    _check(build.core().ns_retention_scan(_ptr(qkv), _ptr(decay), _ptr(state), ctypes.c_longlong(stride), _ptr(qo_indptr), _ptr(state_slots), _ptr(out),
+                                          c_int(state_slots.numel()), c_int(heads), c_int(key_dim), c_int(value_dim), _stream()), "retention_scan")
+    return out
+
+
+def gate_mul(x: torch.Tensor, gate: torch.Tensor, out: torch.Tensor, silu: bool = False) -> torch.Tensor:
+    """out = x * sigmoid(gate), or x * gate * sigmoid(gate) with ``silu``, the gate formed in 32-bit; ``gate`` may be a column
+    slice of wider rows; ``x`` and ``out`` contiguous [tokens, width] (they may be one tensor)."""
+    _gpu(x, gate, out)
+    n, width = x.shape
+    if (not x.is_contiguous() or out.shape != x.shape or not out.is_contiguous() or out.dtype != x.dtype or gate.dtype != x.dtype or gate.shape != x.shape
+            or gate.stride(1) != 1):
+        raise KernelRefused("gate_mul: x and out contiguous [tokens, width], gate [tokens, width] of the same dtype")
+    _check(build.core().ns_gate_mul(_ptr(out), _ptr(x), _ptr(gate), c_int(gate.stride(0)), c_int(n), c_int(width), c_int(1 if silu else 0),
+                                    c_int(_dtype_code(x)), _stream()), "gate_mul")
+    return out
+
+
 def moe_route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, top: int, sel: torch.Tensor, weights: torch.Tensor,
-              logits: torch.Tensor | None = None) -> None:
+              logits: torch.Tensor | None = None, sigmoid: bool = False, correction: torch.Tensor | None = None, groups: int = 1,
+              keep: int = 1) -> None:
     """Router logits z = router h + bias in 32-bit (``router`` float32 [experts, W]); ``sel`` int32 [tokens, top] receives the
     experts with the largest logits in falling order, ``weights`` float32 [tokens, top] the soft-max over those logits.
-    ``logits``: float32 [tokens, experts], receives z (scratch if the caller has no use for it)."""
-    _gpu(h, router, bias, sel, weights, logits)
+    ``logits``: float32 [tokens, experts], receives z (scratch if the caller has no use for it).
+    ``sigmoid``: the scores are s = sigmoid(z), the choice goes by s + ``correction`` (float32 [experts] or None) and the
+    weights are the chosen s themselves.  ``groups`` > 1: only experts of the ``keep`` groups (of experts / groups neighbours)
+    with the largest sums of their two best choice scores can be chosen."""
+    _gpu(h, router, bias, sel, weights, logits, correction)
+    if correction is not None and (not sigmoid or _f32(correction, "correction").numel() != router.shape[0]):
+        raise KernelRefused("moe_route: a correction [experts] belongs to sigmoid scores")
+    if groups < 1 or router.shape[0] % groups or not 1 <= keep <= groups or top > keep * (router.shape[0] // groups):
+        raise KernelRefused(f"moe_route: {router.shape[0]} experts in {groups} groups of which {keep} are kept, {top} chosen")
     _f32(router, "router"), _f32(weights, "weights"), _i32(sel, "sel")
     n, W = h.shape
     experts = router.shape[0]
@@ -1143,11 +1232,12 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, 
             or (bias is not None and _f32(bias, "bias").numel() != experts) or _f32(logits, "logits").shape != (n, experts) or not logits.is_contiguous()):
         raise KernelRefused("moe_route: h [tokens, W], router [experts, W], bias [experts], sel and weights [tokens, top], logits [tokens, experts]")
     _check(build.core().ns_moe_route(_ptr(h), c_int(h.stride(0)), _ptr(router), _ptr(bias), _ptr(logits), _ptr(sel), _ptr(weights), c_int(n), c_int(W),
-                                     c_int(experts), c_int(top), c_int(_dtype_code(h)), _stream()), "moe_route")
+                                     c_int(experts), c_int(top), c_int(1 if sigmoid else 0), _ptr(correction), c_int(groups), c_int(keep),
+                                     c_int(_dtype_code(h)), _stream()), "moe_route")
 
 
 def moe_expert_rows(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
-                    limit: float, alpha: float, act: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+                    limit: float, alpha: float, act: torch.Tensor, out: torch.Tensor, shift: float = 1.0) -> torch.Tensor:
     """out[t, k] = weights[t, k] * expert sel[t, k] of h[t], for few rows: every (token, chosen expert) streams that expert's
     matrices, cut into slices over many workgroups.  ``gate``, ``up`` [experts, ff, W], ``down`` [experts, W, ff] in the dtype
     of ``h``; ``act`` float32 [tokens, top, ff] (scratch); ``out`` float32 [tokens, top, W]."""
@@ -1161,7 +1251,7 @@ def moe_expert_rows(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down:
             or any(t.dtype != h.dtype or not t.is_contiguous() for t in (gate, up, down))):
         raise KernelRefused("moe_expert_rows: gate and up [experts, ff, W], down [experts, W, ff] in the dtype of h; act [tokens, top, ff] and out [tokens, top, W] float32")
     _check(build.core().ns_moe_expert_rows(_ptr(h), c_int(h.stride(0)), _ptr(gate), _ptr(up), _ptr(down), _ptr(sel), _ptr(weights), _ptr(act),
-                                           _ptr(out), c_int(n), c_int(W), c_int(ff), c_int(top), c_float(limit), c_float(alpha),
+                                           _ptr(out), c_int(n), c_int(W), c_int(ff), c_int(top), c_float(limit), c_float(alpha), c_float(shift),
                                            c_int(_dtype_code(h)), _stream()), "moe_expert_rows")
     return out
 
@@ -1172,7 +1262,7 @@ def moe_groups_take(h: torch.Tensor, ff: int) -> bool:
 
 
 def moe_expert_groups(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
-                      limit: float, alpha: float, ints: torch.Tensor, act: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+                      limit: float, alpha: float, ints: torch.Tensor, act: torch.Tensor, out: torch.Tensor, shift: float = 1.0) -> torch.Tensor:
     """The same result for many rows in bfloat16: the pairs are sorted by expert on the device and every expert multiplies
     its rows in tiles on the matrix cores.  ``ints`` int32 [tokens * top + 3 * moe_group_tiles] and ``act`` bfloat16
     [tokens * top, ff] are scratch."""
@@ -1188,12 +1278,12 @@ def moe_expert_groups(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, dow
         raise KernelRefused("moe_expert_groups: bfloat16 operands with sizes in multiples of 8, act [pairs, ff], ints [pairs + 3 tiles]")
     _check(build.core().ns_moe_expert_groups(_ptr(h), c_int(h.stride(0)), _ptr(gate), _ptr(up), _ptr(down), _ptr(sel), _ptr(weights), _ptr(ints),
                                              _ptr(act), _ptr(out), c_int(n), c_int(W), c_int(ff), c_int(top), c_int(experts), c_float(limit),
-                                             c_float(alpha), _stream()), "moe_expert_groups")
+                                             c_float(alpha), c_float(shift), _stream()), "moe_expert_groups")
     return out
 
 
 def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, sel: torch.Tensor, weights: torch.Tensor,
-                limit: float, alpha: float, take) -> torch.Tensor:
+                limit: float, alpha: float, take, shift: float = 1.0) -> torch.Tensor:
     """The chosen experts' weighted outputs, float32 [tokens, top, W], by the kernels that suit the number of rows: with
     fewer (token, expert) pairs than experts every pair streams its expert's matrices; from there on the sorted, tiled
     product reads every matrix at most once.  ``take(shape, dtype)`` gives scratch that lives as long as the result."""
@@ -1204,17 +1294,18 @@ def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: tor
     if n * top >= max(experts, 16) and moe_groups_take(h, ff):
         tiles = int(build.core().ns_moe_group_tiles(c_int(n * top), c_int(experts)))
         return moe_expert_groups(h, gate, up, down, sel, weights, limit, alpha, take((n * top + 3 * tiles,), torch.int32),
-                                 take((n * top, ff), h.dtype), out)
-    return moe_expert_rows(h, gate, up, down, sel, weights, limit, alpha, take((n, top, ff), torch.float32), out)
+                                 take((n * top, ff), h.dtype), out, shift=shift)
+    return moe_expert_rows(h, gate, up, down, sel, weights, limit, alpha, take((n, top, ff), torch.float32), out, shift=shift)
 
 
-def clipped_glu(gu: torch.Tensor, limit: float, alpha: float, out: torch.Tensor) -> torch.Tensor:
-    """out = g sigmoid(alpha g) (u + 1) with g = min(gu[:, :ff], limit), u = clamp(gu[:, ff:], -limit, limit)."""
+def clipped_glu(gu: torch.Tensor, limit: float, alpha: float, out: torch.Tensor, shift: float = 1.0) -> torch.Tensor:
+    """out = g sigmoid(alpha g) (u + shift) with g = min(gu[:, :ff], limit), u = clamp(gu[:, ff:], -limit, limit) (an infinite
+    limit clips nothing)."""
     _gpu(gu, out)
     n, ff = out.shape
     if gu.shape != (n, 2 * ff) or gu.stride(1) != 1 or not out.is_contiguous() or out.dtype != gu.dtype:
         raise KernelRefused("clipped_glu: gu [tokens, 2 ff], out [tokens, ff] of the same dtype")
-    _check(build.core().ns_clipped_glu(_ptr(out), _ptr(gu), c_int(gu.stride(0)), c_int(n), c_int(ff), c_float(limit), c_float(alpha),
+    _check(build.core().ns_clipped_glu(_ptr(out), _ptr(gu), c_int(gu.stride(0)), c_int(n), c_int(ff), c_float(limit), c_float(alpha), c_float(shift),
                                        c_int(_dtype_code(gu)), _stream()), "clipped_glu")
     return out
 
@@ -1304,8 +1395,13 @@ def latent_prep(proj: torch.Tensor, q_norm: torch.Tensor, c_norm: torch.Tensor, 
     if (k_cache.dim() != 4 or k_cache.shape[1:] != (1, page, latent + rot) or v_cache.shape != (k_cache.shape[0], 1, latent, page)
             or k_cache.dtype != proj.dtype or v_cache.dtype != proj.dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
         raise KernelRefused("latent_prep: the pages hold one key of latent + rot channels and one value of latent channels per token")
-    if (q_norm.shape != (q_rank,) or c_norm.shape != (latent,) or q_norm.dtype != proj.dtype or c_norm.dtype != proj.dtype or not q_norm.is_contiguous()
-            or not c_norm.is_contiguous() or cq.shape != (n, q_rank) or cq.dtype != proj.dtype or not cq.is_contiguous()
+    if q_rank == 0:
+        q_norm = cq = None  # no query latent: the layer's queries are projected from its input
+    elif (q_norm.shape != (q_rank,) or q_norm.dtype != proj.dtype or not q_norm.is_contiguous() or cq.shape != (n, q_rank) or cq.dtype != proj.dtype
+          or not cq.is_contiguous()):
+        raise KernelRefused("latent_prep: the query latent's norm weight or output does not fit its size")
+    if (c_norm.shape != (latent,) or c_norm.dtype != proj.dtype
+            or not c_norm.is_contiguous()
             or rot % 2 or inv_freq.numel() < max(1, rot // 2) or token_req.numel() != n or block_table.dim() != 2 or block_table.stride(1) != 1):
         raise KernelRefused("latent_prep: norm weights, outputs or frequencies do not fit the sizes")
     _check(build.core().ns_latent_prep(_ptr(proj), c_int(proj.stride(0)), _ptr(q_norm), _ptr(c_norm), _ptr(inv_freq), c_float(factor), _ptr(cq),
@@ -1460,21 +1556,25 @@ def delta_scan(qkv: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, state: to
     return out
 
 
-def gated_rms(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, out: torch.Tensor,
-              den: torch.Tensor | None = None) -> torch.Tensor:
+def gated_rms(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor | None, eps: float, heads: int, out: torch.Tensor,
+              den: torch.Tensor | None = None, silu: bool = False) -> torch.Tensor:
     """out[t, h, :] = x / sqrt(mean(x^2) + eps) * weight * sigmoid(gate[t, h, :]) with x = o[t, h, :], or o[t, h, :] /
     den[t, h] if ``den`` (float32 [tokens, heads]) is given; ``o`` float32 [tokens, heads * E], ``weight`` float32 [E] (all
-    heads share it) or [heads * E], ``gate`` (may be a column slice) and ``out`` in the model's dtype."""
-    _f32(o, "o"), _f32(weight, "weight")
+    heads share it) or [heads * E] or None (no weight), ``gate`` (may be a column slice) and ``out`` in the model's dtype.
+    ``silu``: the gate is g sigmoid(g) instead of sigmoid(g)."""
+    _f32(o, "o")
+    if weight is not None:
+        _f32(weight, "weight")
     _gpu(gate, out, den)
     n, width = o.shape
-    if (width % heads or weight.numel() not in (width // heads, width) or gate.shape[0] != n or gate.shape[1] < width or gate.stride(1) != 1
+    if (width % heads or (weight is not None and weight.numel() not in (width // heads, width)) or gate.shape[0] != n or gate.shape[1] < width or gate.stride(1) != 1
             or out.shape != (n, width) or not out.is_contiguous() or out.dtype != gate.dtype
             or (den is not None and (_f32(den, "den").shape != (n, heads) or not den.is_contiguous()))):
         raise KernelRefused("gated_rms: operands do not fit heads and value size")
-    per_head = width // heads if (weight.numel() == width and heads > 1) else 0
+    per_head = width // heads if (weight is not None and weight.numel() == width and heads > 1) else 0
     _check(build.core().ns_gated_rms(_ptr(out), _ptr(o), _ptr(gate), c_int(gate.stride(0)), _ptr(weight), c_int(per_head), _ptr(den), c_int(n),
-                                     c_int(heads), c_int(width // heads), c_float(eps), c_int(_dtype_code(gate)), _stream()), "gated_rms")
+                                     c_int(heads), c_int(width // heads), c_float(eps), c_int(1 if silu else 0), c_int(_dtype_code(gate)), _stream()),
+           "gated_rms")
     return out
 
 

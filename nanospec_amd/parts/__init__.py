@@ -1,4 +1,4 @@
-from . import attention, block, delta, dense, latent, memory, moe, norm, parallel, rope, side, swiglu  # noqa: F401  (each registers its parts)
+from . import attention, block, delta, dense, glu, latent, memory, moe, norm, parallel, retention, rope, side, swiglu  # noqa: F401  (each registers its parts)
 from .model import DecoderModel, wanted_tensors
 from .needs import PagedNeed, StateNeed
 from .registry import build, register, registered

@@ -195,8 +195,13 @@ class Attention:
             raise ValueError(f"value_mix={spec.value_mix!r}: use '', 'source' or 'mix'")
         if (spec.bias or spec.whole_norm_eps is not None or spec.value_mix) and not spec.own_kv:
             raise ValueError("biases, whole-projection norms and mixed values belong to a layer with key/value projections of its own")
-        if spec.whole_norm_eps is not None and (spec.qk_norm_eps is not None or self.position.rotary_dim):
-            raise ValueError("a norm over the whole projection stands alone: no per-head unit norm and no rotation beside it")
+        if spec.whole_norm_eps is not None and spec.qk_norm_eps is not None:
+            raise ValueError("a norm over the whole projection stands alone: no per-head unit norm beside it")
+        if (spec.sink_name or spec.out_gate) and not spec.own_kv:
+            raise ValueError("a learned sink and an output gate belong to a layer with key/value projections of its own")
+        if spec.sink_name and spec.sink:
+            raise ValueError("the soft-max has one sink: of score 0, or a learned one")
+        self.sink_logits: torch.Tensor | None = None
         self.head_form = spec.head_norm_eps is not None or spec.value_is_key  # per-head norms with weights, values that are the keys
         if self.head_form and (spec.qk_norm_eps is not None or spec.whole_norm_eps is not None or spec.value_mix or not spec.own_kv):
             raise ValueError("per-head norms with weights and values that are the keys stand beside biases and a rotation only")
@@ -234,6 +239,10 @@ class Attention:
         if s.whole_norm_eps is not None:
             out[q + s.whole_norm_suffix] = ((s.heads * s.head_dim,), "norm")
             out[k + s.whole_norm_suffix] = ((s.kv_heads * s.head_dim,), "norm")
+        if s.sink_name:
+            out[self.prefix + s.sink_name] = ((s.heads,), "around_zero")
+        if s.out_gate:
+            out[self.prefix + s.gate_name] = ((s.heads * s.v_dim, s.hidden), "linear")
         if s.value_mix:
             # (a "source" layer's checkpoint holds the tensor too; it is not used there)
             out[self.prefix + s.value_mix_name] = ((), lambda shape, gen: torch.full(shape, 0.5, device=gen.device)
@@ -245,9 +254,13 @@ class Attention:
         plain = layouts == "both"
         q, k, v, o = self._names
         rows = s.heads * s.head_dim + (s.kv_heads * (s.head_dim + (0 if s.value_is_key else s.v_dim)) if s.own_kv else 0)
+        self.gate_at = rows  # the output gate's logits, if the layer has a gate, are the last columns of the first product
+        stacked = (q,) if not s.own_kv else ((q, k) if s.value_is_key else (q, k, v))
+        if s.out_gate:
+            rows += s.heads * s.v_dim
+            stacked += (self.prefix + s.gate_name,)
         wqkv = torch.empty((rows, s.hidden), dtype=dtype, device=device)
         at = 0
-        stacked = (q,) if not s.own_kv else ((q, k) if s.value_is_key else (q, k, v))
         for name in stacked:
             t = get(name)
             wqkv[at : at + t.shape[0]].copy_(t)
@@ -257,6 +270,8 @@ class Attention:
         self._form = dict(interleaved=bool(getattr(self.position, "interleaved", False)), factor=float(getattr(self.position, "factor", 1.0)))
         to = lambda name: get(name).to(device=device, dtype=dtype).contiguous()
         if s.bias:
+            if s.out_gate:
+                raise ValueError("an output gate beside biased projections is not built")
             self.qkv_bias = torch.cat([to(name + s.bias_suffix) for name in stacked]).contiguous()
             self.out_bias = to(o + s.bias_suffix)
         if s.head_norm_eps is not None:
@@ -265,6 +280,8 @@ class Attention:
             self.q_norm, self.k_norm = to(q + s.whole_norm_suffix), to(k + s.whole_norm_suffix)
         if s.value_mix == "mix":
             self.v_mix = to(self.prefix + s.value_mix_name).reshape(1)
+        if s.sink_name:
+            self.sink_logits = get(self.prefix + s.sink_name).to(device=device, dtype=torch.float32).contiguous()
         if s.general:
             # the general path: one product for what the layer projects, then norm / cache write and attention as kernels
             self.wqkv_rope = None
@@ -362,6 +379,13 @@ class Attention:
             ops.head_norm_rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq if pos.rotary_dim else None, cache.k, cache.v,
                                         s.heads, s.kv_heads, s.head_dim, s.v_dim, s.head_norm_eps or 0.0, pos.rotary_dim, bias=self.qkv_bias,
                                         q_weight=self.q_head_norm, k_weight=self.k_head_norm, value_is_key=s.value_is_key, **self._form)
+        elif s.whole_norm_eps is not None and pos.rotary_dim:
+            # a norm over the whole of q and of k, then the rotation, then the pages
+            if s.bias or s.value_mix:
+                raise ops.KernelRefused("rotation behind a whole-projection norm together with biases or mixed values is not built")
+            ops.whole_norm_kv_write(qkv, ctx.positions, ctx.token_req, table, cache.k, cache.v, s.heads, s.kv_heads, s.head_dim, s.v_dim,
+                                    s.whole_norm_eps, q_weight=self.q_norm, k_weight=self.k_norm, inv_freq=pos.inv_freq,
+                                    rotary_dim=pos.rotary_dim, **self._form)
         elif pos.rotary_dim:
             if s.qk_norm_eps is not None or s.v_dim != s.head_dim or not s.own_kv:
                 raise ops.KernelRefused("rotation together with unit-RMS queries and keys, another value size or borrowed keys is not built")
@@ -383,20 +407,22 @@ class Attention:
             ops.unit_kv_write(qkv, ctx.positions, ctx.token_req, table, cache.k, cache.v, s.heads, s.kv_heads, s.head_dim, s.v_dim,
                               s.qk_norm_eps, own_kv=s.own_kv)
         att = ctx.arena.take((n, s.heads * s.v_dim), x.dtype)
-        if s.v_dim == s.head_dim and not s.slope_exp and ops.mfma_attention_takes(x.dtype, s.head_dim, cache.k.shape[2]):
+        if s.v_dim == s.head_dim and not s.slope_exp and not s.sink_name and ops.mfma_attention_takes(x.dtype, s.head_dim, cache.k.shape[2]):
             # bfloat16 on the matrix cores: the tile kernels honour chunks, capped scores and the sink
             for plan in launch_plans(ctx, s.heads // s.kv_heads, s.kv_heads, s.head_dim, span=s.chunk):
                 ops.attention_mfma(qkv, att, cache.k, cache.v, plan.tiles, table, s.heads, s.kv_heads, s.head_dim, s.softmax_scale,
                                    window=s.window, hp=plan.hp, splits=plan.splits, workspace=plan.workspace, qt=plan.qt, coop=plan.coop,
                                    chunk=s.chunk, cap=s.score_cap, sink=s.sink)
-        elif not (s.chunk or s.score_cap or s.sink) and ops.wide_attention_takes(x.dtype, s.head_dim, s.v_dim, cache.k.shape[2]):
+        elif not (s.chunk or s.score_cap or s.sink or s.sink_name) and ops.wide_attention_takes(x.dtype, s.head_dim, s.v_dim, cache.k.shape[2]):
             # bfloat16, values of another size than the keys or a bias by distance: the two-size matrix-core kernel
             wide_attention(ctx, qkv, att, cache, table, s.heads, s.kv_heads, s.head_dim, s.v_dim, s.softmax_scale, window=s.window,
                            slope_exp=s.slope_exp)
         else:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads, s.head_dim,
                                   s.softmax_scale, window=s.window, v_dim=s.v_dim, chunk=s.chunk, cap=s.score_cap, sink=s.sink,
-                                  slope_exp=s.slope_exp)
+                                  slope_exp=s.slope_exp, sink_logits=self.sink_logits)
+        if s.out_gate:
+            ops.gate_mul(att, qkv[:, self.gate_at : self.gate_at + s.heads * s.v_dim], out=att)
         if residual is not None and self.out_bias is None:
             return self.wo.into_residual(att, residual, arena=ctx.arena, plain_copy=not ctx.captured)
         y = self.wo(att, out=out if out is not None else ctx.arena.take((n, s.hidden), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)

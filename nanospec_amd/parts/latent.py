@@ -37,6 +37,9 @@ class LatentAttention:
         if spec.rot_dim % 2:
             raise ValueError(f"rot_dim={spec.rot_dim} must be even")
         self.first: LinearWeight | None = None
+        self.sink_logits: torch.Tensor | None = None
+        if not spec.q_rank and spec.gate:
+            raise ValueError("a latent-attention layer without a query latent has no gate per head")
 
     @property
     def _n(self) -> dict:
@@ -46,14 +49,17 @@ class LatentAttention:
     def wanted(self) -> dict:
         s, n = self.spec, self._n
         out = {
-            n["dq"]: ((s.q_rank, s.hidden), "linear"), n["dq_norm"]: ((s.q_rank,), "norm"),
-            n["uq"]: ((s.heads * (s.head_dim + s.rot_dim), s.q_rank), "linear"),
+            n["uq"]: ((s.heads * (s.head_dim + s.rot_dim), s.q_rank or s.hidden), "linear"),
             n["dkv"]: ((s.kv_rank + s.rot_dim, s.hidden), "linear"), n["dkv_norm"]: ((s.kv_rank,), "norm"),
             n["uk"]: ((s.heads * s.head_dim, s.kv_rank), "linear"), n["uv"]: ((s.heads * s.value_dim, s.kv_rank), "linear"),
             n["o"]: ((s.hidden, s.heads * s.value_dim), "linear"),
         }
+        if s.q_rank:
+            out.update({n["dq"]: ((s.q_rank, s.hidden), "linear"), n["dq_norm"]: ((s.q_rank,), "norm")})
         if s.gate:
             out[n["g"]] = ((s.heads, s.hidden), "linear")
+        if s.sink_name:
+            out[self.prefix + s.sink_name] = ((s.heads,), "around_zero")
         return out
 
     def load(self, get, dtype, device, layouts: str = "both") -> None:
@@ -61,13 +67,18 @@ class LatentAttention:
         plain = layouts == "both"
         to = lambda name: get(name).to(device=device, dtype=dtype).contiguous()
         # one product for everything that reads the layer's input: [W_dq; W_dkv; W_g]
-        self.first = LinearWeight(torch.cat([to(n["dq"]), to(n["dkv"])] + ([to(n["g"])] if s.gate else [])).contiguous(), keep_plain=plain)
-        self.dq_norm, self.dkv_norm = to(n["dq_norm"]), to(n["dkv_norm"])
-        self.uq = LinearWeight(to(n["uq"]), keep_plain=plain)
+        # (without a query latent the queries' matrix takes the place of W_dq in it, and there is no second product)
+        self.q_cols = s.q_rank or s.heads * (s.head_dim + s.rot_dim)
+        self.first = LinearWeight(torch.cat([to(n["dq"] if s.q_rank else n["uq"]), to(n["dkv"])] + ([to(n["g"])] if s.gate else [])).contiguous(),
+                                  keep_plain=plain)
+        self.dq_norm, self.dkv_norm = (to(n["dq_norm"]) if s.q_rank else None), to(n["dkv_norm"])
+        self.uq = LinearWeight(to(n["uq"]), keep_plain=plain) if s.q_rank else None
+        if s.sink_name:
+            self.sink_logits = get(self.prefix + s.sink_name).to(device=device, dtype=torch.float32).contiguous()
         # the two per-head matrices, each in the layout its kernel walks: on the matrix cores (bfloat16, sizes that fit) every
         # head's matrix as [out, in] rows; otherwise as the plain kernels of ``csrc/latent.hip`` read them
         D, R, E, C = s.head_dim, s.rot_dim, s.value_dim, s.kv_rank
-        self._mfma_q = ops.headwise_takes(dtype, C, D, D + R, C + R) and s.hidden % 8 == 0 and s.q_rank % 8 == 0
+        self._mfma_q = ops.headwise_takes(dtype, C, D, D + R, C + R) and s.hidden % 8 == 0 and s.q_rank % 8 == 0 and self.q_cols % 8 == 0
         self._mfma_o = ops.headwise_takes(dtype, E, C, C, E)
         uk, uv = to(n["uk"]), to(n["uv"])
         self.uk = uk.view(s.heads, D, C).transpose(1, 2).contiguous() if self._mfma_q else uk  # [heads, latent, dim] | [heads * dim, latent]
@@ -97,21 +108,27 @@ class LatentAttention:
         take = ctx.arena.take
         table = ctx.block_tables[cache.group]
         proj = self.first(x, out=take((n, self.first.n), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
-        cq = take((n, s.q_rank), x.dtype)
         gate = take((n, H), torch.float32) if s.gate else None
-        ops.latent_prep(proj, self.dq_norm, self.dkv_norm, pos.inv_freq, self._factor, ctx.positions, ctx.token_req, table, cache.k, cache.v,
-                        s.q_rank, C, R, H if s.gate else 0, s.norm_eps, cq, gate)
-        q = self.uq(cq, out=take((n, H * (D + R)), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
+        if s.q_rank:
+            cq = take((n, s.q_rank), x.dtype)
+            ops.latent_prep(proj, self.dq_norm, self.dkv_norm, pos.inv_freq, self._factor, ctx.positions, ctx.token_req, table, cache.k, cache.v,
+                            s.q_rank, C, R, H if s.gate else 0, s.norm_eps, cq, gate)
+            q = self.uq(cq, out=take((n, H * (D + R)), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
+        else:
+            # the queries are the first columns of the product; the rest of a row is [latent | rotated part]
+            ops.latent_prep(proj[:, self.q_cols :], None, self.dkv_norm, pos.inv_freq, self._factor, ctx.positions, ctx.token_req, table, cache.k,
+                            cache.v, 0, C, R, 0, s.norm_eps, None, None)
+            q = proj[:, : self.q_cols]
         q_lat = take((n, H * (C + R)), x.dtype)
         if self._mfma_q:
             ops.headwise_product(q, D + R, self.uk, q_lat, C + R)
         ops.latent_q_absorb(q, None if self._mfma_q else self.uk, pos.inv_freq, self._factor, ctx.positions, H, D, R, C, out=q_lat)
         o_lat = take((n, H * C), x.dtype)
-        if ops.wide_attention_takes(x.dtype, C + R, C, cache.k.shape[2]):
+        if self.sink_logits is None and ops.wide_attention_takes(x.dtype, C + R, C, cache.k.shape[2]):
             wide_attention(ctx, q_lat, o_lat, cache, table, H, 1, C + R, C, s.softmax_scale, window=s.window)
         else:
             ops.attention_generic(q_lat, o_lat, cache.k, cache.v, ctx.token_req, ctx.positions, table, H, 1, C + R, s.softmax_scale,
-                                  window=s.window, v_dim=C)
+                                  window=s.window, v_dim=C, sink_logits=self.sink_logits)
         att = take((n, H * E), x.dtype)
         if self._mfma_o:
             ops.headwise_product(o_lat, C, self.uv, att, E, gate=gate)

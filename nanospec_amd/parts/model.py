@@ -28,6 +28,9 @@ def wanted_tensors(spec, layers=None) -> dict:
         out[pair.name] = ((pair.buckets + 1, spec.hidden), "embedding")
     for layer in layers:
         out.update(layer.wanted())
+    passes = getattr(spec, "passes", None)
+    if passes is not None:
+        out[passes.name] = ((passes.times, spec.hidden), "embedding")
     out.update(registry.build("norm", spec.final_norm, spec.final_norm_name).wanted())
     out[spec.head_name] = ((spec.vocab_size, spec.hidden), "linear")
     return out
@@ -56,6 +59,11 @@ class DecoderModel:
         if self.pair is not None and not spec.streams:
             raise ValueError("a pair embedding is built for models that carry 32-bit streams")
         self.pair_table: torch.Tensor | None = None
+        # a range of layers that runs several times: what each pass adds to the stream in front of it (``LayerCall.enters``)
+        self.passes = getattr(spec, "passes", None)
+        if self.passes is not None and not spec.streams:
+            raise ValueError("passes over a range of layers are built for models that carry 32-bit streams")
+        self.pass_rows: torch.Tensor | None = None
         # state of fixed size per request that belongs to no layer: name -> StateNeed (the cache storage keeps a tensor
         # [slots, *shape] for each, zeroed at admission, and the step's context hands them over as ``ctx.model_state``)
         self.state_needs = {self.LAST_TOKEN: StateNeed((1,), torch.int32)} if self.pair is not None else {}
@@ -122,6 +130,8 @@ class DecoderModel:
         self.final_norm.load(get, dtype, device)
         if self.pair is not None:
             self.pair_table = get(self.pair.name).to(device=device, dtype=dtype).contiguous()
+        if self.passes is not None:
+            self.pass_rows = get(self.passes.name).to(device=device, dtype=dtype).contiguous()
         if spec.streams:
             self._ones = torch.ones(spec.streams, dtype=torch.float32, device=device)
         # whoever runs the model works on a stream of their own: everything that loading enqueued (copies, re-laying of
@@ -169,6 +179,17 @@ class DecoderModel:
             pending = None
             carry = ctx.arena.take((n, self.spec.hidden), self.dtype)
             for i, call in enumerate(self.spec.run_order):
+                if call.enters is not None:
+                    # a pass starts: what the layer before left unwritten goes into the streams, then the embedding's output
+                    # (every pass but the first) and the pass's own row, each added in 32-bit
+                    if pending is not None:
+                        ops.stream_step(resid, pending)
+                        pending = None
+                    again = self.passes.add_embedding and call.enters > 0
+                    if again and self.pair is not None:
+                        raise ops.KernelRefused("a pass that adds the embedding's output again beside a pair embedding is not built")
+                    ops.stream_add_rows(resid, self.embed if again else None, ctx.token_ids if again else None, self.pass_rows[call.enters],
+                                        scale=self.spec.embed_scale)
                 pending = self.layers[call.layer].forward(ctx, resid, pending, caches[i], call.cache_from is None, carry)
                 if self.layer_probe is not None:
                     total = torch.empty((n, self.spec.hidden), dtype=torch.float32, device=resid.device)
