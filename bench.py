@@ -274,9 +274,43 @@ def padetar_config(shape: dict, layers: int | None = None):
                                   "token_side": {"dim": 256}, "layers": [entry] * n})
 
 
+# Sizes for ``--design fimilorn``: the Fimilorn design at the widths, depths and head counts of the Llama shapes above.  The
+# layers take turns: attention (the shape's heads and key/value heads, the whole head rotated, a norm over the whole of q and
+# of k, learned sinks, an output gate), latent attention (the shape's heads with head_dim unrotated and head_dim / 2 rotated
+# channels, a latent of 512, windows of 1,024, learned sinks), retention (width / 256 heads of 128 key and 256 value channels).
+# The first layer's feed-forward is the clipped dense one of the shape's inner size; every other is 32 experts of an eighth of
+# it in 8 groups of which 4 are kept, four experts a token, beside a shared expert of half the inner size.  The first three
+# layers run twice, and the model has three layers fewer than the shape, so that a token passes as many layers.
+def fimilorn_config(shape: dict, layers: int | None = None):
+    from nanospec_amd.config import FimilornConfig
+
+    n = max(4, (layers or shape["num_hidden_layers"]) - 3)
+    heads, kvh, hd, ff, width = (shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"], shape["intermediate_size"],
+                                 shape["hidden_size"])
+    rh = width // 256
+    mixers = [
+        ("attention", dict(heads=heads, kv_heads=kvh, dim=hd, vdim=hd, scale=hd ** -0.5, rot={"base": 1e6, "dims": hd})),
+        ("latent_attention", dict(heads=heads, dim=hd, rot_dim=hd // 2, vdim=hd, kv_rank=512, scale=(hd + hd // 2) ** -0.5, mask={"size": 1024},
+                                  rot={"base": 1e6, "dims": hd // 2})),
+        ("retention", dict(heads=rh, dim=128, vdim=256, decay=[1.0 - 2.0 ** (-5 - h % 8) for h in range(rh)], rot={"base": 1e4, "dims": 128})),
+    ]
+    moe = {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 32, "top": 4, "groups": {"count": 8, "keep": 4}}, "shared": {"ff": ff // 2}}
+    entries = [{"type": mixers[i % 3][0], "mixer": mixers[i % 3][1], "mlp": {"kind": "dense", "ff": ff, "limit": 7.0} if i == 0 else moe}
+               for i in range(n)]
+    return FimilornConfig.from_hf({"architecture": "Fimilorn", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6},
+                                   "loop": {"start": 0, "stop": 3, "times": 2}, "layers": entries})
+
+
+DESIGNS = {"vuzelix": vuzelix_config, "fetitar": fetitar_config, "padetar": padetar_config, "fimilorn": fimilorn_config}
+# the existing model that a design is closest to, measured beside it as well (Llama always is): Padetar, like Fimilorn, has a
+# mixture of experts with a shared expert and a recurrent mixer beside soft-max attention over a 32-bit stream
+CLOSEST = {"fimilorn": "padetar"}
+
+
 def design_compare(a) -> int:
-    """``--design NAME``: prefill and decode throughput of that design beside the Llama model of the same shape,
-    one JSON line.  The default workload and its output are not touched by this option."""
+    """``--design NAME``: prefill and decode throughput of that design beside the Llama model of the same shape (and
+    beside the existing design it is closest to, if ``CLOSEST`` names one), one JSON line.  The default workload and its
+    output are not touched by this option."""
     import types
 
     import torch
@@ -291,10 +325,11 @@ def design_compare(a) -> int:
     llama = LlamaConfig.from_hf(dict(model_type="llama", **{k: v for k, v in shape.items() if k != "rope_scaling"},
                                      rope_scaling=dict(rope_type="llama3", **shape["rope_scaling"])))
     design = a.design
-    vz = {"vuzelix": vuzelix_config, "fetitar": fetitar_config, "padetar": padetar_config}[design](shape)
+    vz = DESIGNS[design](shape)
     out = {}
     k = min(a.steps, 128)
-    for name, cfg in (("llama", llama), (design, vz)):
+    beside = [(CLOSEST[design], DESIGNS[CLOSEST[design]](shape))] if design in CLOSEST else []
+    for name, cfg in (("llama", llama), *beside, (design, vz)):
         model = random_model(cfg, seed=0, dtype=dtype, on_device=True)
         facts = types.SimpleNamespace(vocab_size=shape["vocab_size"])
         row = {}
@@ -314,6 +349,9 @@ def design_compare(a) -> int:
                       "unit": "tok/s", "n_gpus": 1, "dtype": a.dtype, "data": "synthetic: random weights, uniform random token ids",
                       "config": {"shape": SHAPE_NAMES[a.shape], "layers": shape["num_hidden_layers"], "hidden": shape["hidden_size"],
                                  f"{design}_layers": layers, "streams": getattr(vz, "streams", 1), "page_size": 16, "decode_steps": k},
+                      **{name: out[name] for name, _ in beside},
+                      **{f"{design}_over_{name}": {key: round(out[design][key] / out[name][key], 3) for key in out[name] if key.endswith("tok_s")}
+                         for name, _ in beside},
                       "llama": out["llama"], design: out[design], f"{design}_over_llama": ratio}), flush=True)
     return 0
 
@@ -334,7 +372,7 @@ def main() -> int:
                     help="instead of the benchmark: continuous batching of this many requests (prompts of 16 to 1,024 tokens, 128 new "
                          "tokens each, prompts in portions of 512)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="the benchmark's shape is 8b; the others are for profiles")
-    ap.add_argument("--design", default=None, choices=["vuzelix", "fetitar", "padetar"],
+    ap.add_argument("--design", default=None, choices=sorted(DESIGNS),
                     help="instead of the benchmark: prefill and decode of this design beside the Llama model of the same --shape")
     a = ap.parse_args()
     if a.gpus != 1:

@@ -67,7 +67,8 @@ struct AttnParams {
   float scale_log2;  // softmax scale * log2(e)
   // Options, read only by the kernels instantiated with OPT (every other kernel is compiled as if they did not exist):
   int chunk;         // > 0: a query sees no key before the start of its own chunk of this many positions
-  int sink;          // the soft-max's denominator holds one more term of score 0
+  int sink;          // the soft-max's denominator holds one more term of score 0 ...
+  const float* sink_logits;  // ... or, if given, of the learned score sink_logits[head], which is not scaled
   float cap;         // > 0: a score s (after the scale) becomes cap * tanh(s / cap); scale_log2 is then log2(e) alone
   float cap_pre;     // softmax scale / cap
 };
@@ -436,7 +437,7 @@ __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
     if (a.splits == 1) {
       const size_t col = (size_t)(q0 + t0 + tt) * a.heads + head;
       if constexpr (OPT) {
-        if (a.sink) lsum[u] += fast_exp2(-m[u] * a.scale_log2);  // the term of score 0, in the units of the column's maximum
+        if (a.sink) lsum[u] += fast_exp2((a.sink_logits ? a.sink_logits[head] * 1.4426950408889634f : 0.f) - m[u] * a.scale_log2);  // the sink's term, in the units of the column's maximum
       }
       const float inv = 1.f / lsum[u];
 #pragma unroll
@@ -995,7 +996,7 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
       if (a.splits == 1) {
         const size_t col = (size_t)(q0 + t0 + u * 16 + c) * a.heads + head;
         if constexpr (OPT) {
-          if (a.sink) lsum[u] += fast_exp2(-m[u] * a.scale_log2);  // the term of score 0, in the units of the column's maximum
+          if (a.sink) lsum[u] += fast_exp2((a.sink_logits ? a.sink_logits[head] * 1.4426950408889634f : 0.f) - m[u] * a.scale_log2);  // the sink's term, in the units of the column's maximum
         }
         const float inv = 1.f / lsum[u];
 #pragma unroll
@@ -1025,7 +1026,7 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
 // results are addressed by tile, so nothing here waits for the tile descriptor except the final store.
 __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                                                          const float* __restrict__ part_ml, const int* __restrict__ tiles,
-                                                         int heads, int tile_tokens, int splits, int sink) {
+                                                         int heads, int tile_tokens, int splits, int sink, const float* __restrict__ sink_logits) {
   const int tile = blockIdx.x, head = blockIdx.y, tt = blockIdx.z;
   const int lane = threadIdx.x;
   const size_t pcol = ((size_t)tile * tile_tokens + tt) * heads + head;
@@ -1047,7 +1048,7 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ ou
   float l = ls * wgt;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
-  if (sink) l += exp2f(-mstar);  // the term of score 0 (the ranges' maxima are in the exponent's units)
+  if (sink) l += exp2f((sink_logits ? sink_logits[head] * 1.4426950408889634f : 0.f) - mstar);  // the sink's term (the ranges' maxima are in the exponent's units)
   const float inv = 1.f / l;
   float acc[PER];
 #pragma unroll
@@ -1103,7 +1104,8 @@ extern "C" int ns_attn_prompt_form(void) { return prompt_form(); }
 extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache,
                             const void* v_cache, const int* tiles, const int* block_table, int table_stride, int n_tiles,
                             int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale, int qt,
-                            int coop, long pool_pages, int chunk, float cap, int sink, hipStream_t stream) {
+                            int coop, long pool_pages, int chunk, float cap, int sink, const float* sink_logits, hipStream_t stream) {
+  if (sink_logits) sink = 1;
   if (chunk < 0 || cap < 0.f) return NS_ERR_BAD_ARG;
   if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size != PS || window < 0 ||
       splits < 1 || splits > 64 || (q_stride & 7) || ((uintptr_t)tiles & 15))
@@ -1124,7 +1126,7 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   a.scale_log2 = scale * 1.4426950408889634f;
   // chunks, capped scores and a sink are honoured by the kernels that walk tiles without sharing keys through LDS
   const bool opt = chunk > 0 || cap > 0.f || sink != 0;
-  a.chunk = chunk; a.sink = sink; a.cap = cap; a.cap_pre = cap > 0.f ? scale / cap : 0.f;
+  a.chunk = chunk; a.sink = sink; a.sink_logits = sink_logits; a.cap = cap; a.cap_pre = cap > 0.f ? scale / cap : 0.f;
   if (cap > 0.f) a.scale_log2 = 1.4426950408889634f;  // the scale is applied where the scores are capped
   const int G = heads / kv_heads;
   const long items = (long)n_tiles * splits * kv_heads * ((G + hp - 1) / hp);
@@ -1170,6 +1172,6 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   if (heads > 65535) return NS_ERR_BAD_ARG;
   const int tile_tokens = qt * 16 / hp;
   attn_reduce_kernel<<<dim3(n_tiles, heads, tile_tokens), 64, 0, stream>>>((bf16_t*)out, (const float*)part_o, (const float*)part_ml,
-                                                                           tiles, heads, tile_tokens, splits, sink);
+                                                                           tiles, heads, tile_tokens, splits, sink, sink_logits);
   return ns_launch_status();
 }

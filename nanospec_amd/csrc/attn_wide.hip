@@ -49,6 +49,7 @@ struct WideParams {
   float scale_log2;  // softmax scale * log2(e)
   float slope_exp;   // see above; 0: none
   float inv_scale;   // 1 / softmax scale: the slope in the units of the unscaled scores
+  const float* sink_logits;  // null, or [heads]: the soft-max's denominator holds one more term exp(sink_logits[head]), not scaled
 };
 
 __device__ __forceinline__ int wmax_i(int v) {
@@ -361,6 +362,7 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(WideParams a) {
   // o[dt][j] is channel 16 dt + 4 g + j of column c
   if (a.splits == 1) {
     const size_t col = (size_t)(q0 + ti) * a.heads + head;
+    if (a.sink_logits) lsum += exp2f(a.sink_logits[head] * 1.4426950408889634f - m * a.scale_log2);  // the sink's term, in the units of the column's maximum
     const float inv = 1.f / lsum;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
@@ -384,7 +386,7 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(WideParams a) {
 // add the ranges in order.
 __global__ __launch_bounds__(64) void attn_wide_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                                                               const float* __restrict__ part_ml, const int* __restrict__ tiles,
-                                                              int heads, int tile_tokens, int splits) {
+                                                              int heads, int tile_tokens, int splits, const float* __restrict__ sink_logits) {
   const int tile = blockIdx.x, head = blockIdx.y, tt = blockIdx.z;
   const int lane = threadIdx.x;
   const size_t pcol = ((size_t)tile * tile_tokens + tt) * heads + head;
@@ -404,6 +406,7 @@ __global__ __launch_bounds__(64) void attn_wide_reduce_kernel(bf16_t* __restrict
   float l = ls * wgt;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+  if (sink_logits) l += exp2f(sink_logits[head] * 1.4426950408889634f - mstar);  // the sink's term (the ranges' maxima are in the exponent's units)
   const float inv = 1.f / l;
   constexpr int PER = (VD + 63) / 64;
   const float* po = part_o + pcol * splits * VD;
@@ -442,7 +445,7 @@ extern "C" int ns_attn_wide_page_size() { return PS; }
 // and part_ml n_tiles * T * heads * splits * 2.
 extern "C" int ns_attn_wide(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache, const void* v_cache,
                             const int* tiles, const int* block_table, int table_stride, int n_tiles, int heads, int kv_heads, int page_size,
-                            int hp, int splits, int window, float scale, int qt, float slope_exp, hipStream_t stream) {
+                            int hp, int splits, int window, float scale, int qt, float slope_exp, const float* sink_logits, hipStream_t stream) {
   if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size != PS || window < 0 || splits < 1 || splits > 64 ||
       (q_stride & 7) || ((uintptr_t)tiles & 15) || slope_exp < 0.f)
     return NS_ERR_BAD_ARG;
@@ -456,7 +459,7 @@ extern "C" int ns_attn_wide(void* out, void* part_o, void* part_ml, const void* 
   a.q_stride = q_stride; a.table_stride = table_stride; a.n_tiles = n_tiles; a.heads = heads; a.kv_heads = kv_heads;
   a.hp = hp; a.splits = splits; a.window = window; a.qt = qt;
   a.scale_log2 = scale * 1.4426950408889634f;
-  a.slope_exp = slope_exp; a.inv_scale = 1.f / scale;
+  a.slope_exp = slope_exp; a.inv_scale = 1.f / scale; a.sink_logits = sink_logits;
   const int G = heads / kv_heads;
   const long items = (long)n_tiles * qt * splits * kv_heads * ((G + hp - 1) / hp);
   const long blocks = (items + 3) / 4;
@@ -474,6 +477,6 @@ extern "C" int ns_attn_wide(void* out, void* part_o, void* part_ml, const void* 
   if (st != NS_OK || splits == 1) return st;
   const int tile_tokens = qt * 16 / hp;
   attn_wide_reduce_kernel<<<dim3(n_tiles, heads, tile_tokens), 64, 0, stream>>>((bf16_t*)out, (const float*)part_o, (const float*)part_ml,
-                                                                                tiles, heads, tile_tokens, splits);
+                                                                                tiles, heads, tile_tokens, splits, sink_logits);
   return ns_launch_status();
 }

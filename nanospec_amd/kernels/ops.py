@@ -730,7 +730,8 @@ TILE_INTS = 8  # ints per attention tile descriptor: request, first token, first
 def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_heads: int, head_dim: int, scale: float,
                    window: int = 0, hp: int = 1, splits: int = 1,
                    workspace: tuple[torch.Tensor, torch.Tensor] | None = None, qt: int = 1, coop: bool = False,
-                   short_offsets: bool = True, chunk: int = 0, cap: float = 0.0, sink: bool = False) -> torch.Tensor:
+                   short_offsets: bool = True, chunk: int = 0, cap: float = 0.0, sink: bool = False,
+                   sink_logits: torch.Tensor | None = None) -> torch.Tensor:
     """bfloat16 attention on the matrix cores for the tiles described in ``tiles`` (int32 [n_tiles, 8]: request, first
     token of the tile among the request's tokens of this step, row of the request's first token in ``q``, tokens of the
     request in this step, keys after this step, three zeros).  ``hp`` heads of a group times 16/hp tokens make a tile;
@@ -739,9 +740,11 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
     waves of a workgroup share each tile and range (for decode, where a wave's chain of loads is what takes the time); with
     ``qt`` = 2 it asks for workgroups of one set of four waves instead of two (for long rows of keys).  A pool within
     4 GiB is addressed with 32-bit offsets from its start; ``short_offsets`` = False keeps every address 64 bits wide
-    whatever the pool's size (the form that larger pools take).  ``chunk``, ``cap``, ``sink``: as for
+    whatever the pool's size (the form that larger pools take).  ``chunk``, ``cap``, ``sink``, ``sink_logits``: as for
     ``attention_generic``; with any of them the tiles are walked by the kernels that do not share keys through LDS."""
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim)
+    if sink_logits is not None and _f32(sink_logits, "sink_logits").numel() != heads:
+        raise KernelRefused(f"attention_mfma: sink_logits holds one float32 value for each of the {heads} heads")
     if not mfma_attention_takes(q.dtype, head_dim, page):
         raise KernelRefused(f"attention_mfma takes bfloat16, head sizes that are multiples of 16 up to 256 and page sizes that are "
                             f"powers of two from 4; got {q.dtype}, head size {head_dim}, page {page}")
@@ -767,7 +770,7 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
                             _ptr(block_table), c_int(block_table.stride(0)), c_int(n_tiles), c_int(heads), c_int(kv_heads),
                             c_int(page), c_int(hp), c_int(splits), c_int(window), c_float(scale), c_int(qt), c_int(1 if coop else 0),
                             ctypes.c_long(k_cache.shape[0] if short_offsets else 0), c_int(chunk), c_float(cap), c_int(1 if sink else 0),
-                            _stream()),
+                            _ptr(sink_logits), _stream()),
            "attention_mfma")
     return out
 
@@ -779,12 +782,14 @@ def wide_attention_takes(dtype, head_dim: int, v_dim: int, page_size: int) -> bo
 
 def attention_wide(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_heads: int, head_dim: int, v_dim: int, scale: float,
                    window: int = 0, hp: int = 1, splits: int = 1, workspace: tuple[torch.Tensor, torch.Tensor] | None = None, qt: int = 1,
-                   slope_exp: float = 0.0) -> torch.Tensor:
+                   slope_exp: float = 0.0, sink_logits: torch.Tensor | None = None) -> torch.Tensor:
     """bfloat16 attention on the matrix cores for keys of ``head_dim`` and values of ``v_dim`` channels (multiples of 16 up
     to 1,024 and 512), over the tiles of ``tiles`` (as for ``attention_mfma``): ``hp`` heads of a group times 16/hp tokens
     are one wave's columns, ``qt`` such sets of tokens a tile.  ``splits`` > 1 cuts every tile's keys into ranges and needs
-    ``workspace`` = (part_o, part_ml) float32 tensors.  ``slope_exp``: as for ``attention_generic``."""
+    ``workspace`` = (part_o, part_ml) float32 tensors.  ``slope_exp``, ``sink_logits``: as for ``attention_generic``."""
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim, v_dim)
+    if sink_logits is not None and _f32(sink_logits, "sink_logits").numel() != heads:
+        raise KernelRefused(f"attention_wide: sink_logits holds one float32 value for each of the {heads} heads")
     if not wide_attention_takes(q.dtype, head_dim, v_dim, page):
         raise KernelRefused(f"attention_wide takes bfloat16, key sizes that are multiples of 16 up to 1024, value sizes up to 512 and page "
                             f"sizes that are powers of two from 4; got {q.dtype}, sizes {head_dim} and {v_dim}, page {page}")
@@ -806,8 +811,8 @@ def attention_wide(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
     lib = build.attn_wide(head_dim, v_dim, page)
     _check(lib.ns_attn_wide(_ptr(out), _ptr(po), _ptr(pm), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(tiles),
                             _ptr(block_table), c_int(block_table.stride(0)), c_int(n_tiles), c_int(heads), c_int(kv_heads), c_int(page),
-                            c_int(hp), c_int(splits), c_int(window), c_float(scale), c_int(qt), c_float(slope_exp), _stream()),
-           "attention_wide")
+                            c_int(hp), c_int(splits), c_int(window), c_float(scale), c_int(qt), c_float(slope_exp), _ptr(sink_logits),
+                            _stream()), "attention_wide")
     return out
 
 

@@ -138,7 +138,7 @@ WIDE_RANGE_KEYS = 64  # the fewest keys that a range of a row's keys is worth a 
 
 
 def wide_attention(ctx, q, out, cache, table, heads: int, kv_heads: int, head_dim: int, v_dim: int, scale: float, window: int = 0,
-                   slope_exp: float = 0.0):
+                   slope_exp: float = 0.0, sink_logits=None):
     """Launch ``ops.attention_wide`` (keys and values of two sizes on the matrix cores) over the tile lists of the batch:
     prompt portions as sets of 16 tokens of one head, decode rows with up to 16 heads of a group in one wave's columns and
     the keys cut into ranges until the launch fills the GPU (an item of that kernel is one wave)."""
@@ -156,7 +156,7 @@ def wide_attention(ctx, q, out, cache, table, heads: int, kv_heads: int, head_di
             cols = chunk_tiles.shape[0] * TilePlan.TOKENS * heads
             ws = (take((cols * splits * v_dim,), torch.float32), take((cols * splits * 2,), torch.float32))
         ops.attention_wide(q, out, cache.k, cache.v, chunk_tiles, table, heads, kv_heads, head_dim, v_dim, scale, window=window, hp=1,
-                           splits=splits, workspace=ws, qt=qt, slope_exp=slope_exp)
+                           splits=splits, workspace=ws, qt=qt, slope_exp=slope_exp, sink_logits=sink_logits)
     if decode_tiles.shape[0]:
         hp = 1
         while hp < min(group, 16):
@@ -171,7 +171,7 @@ def wide_attention(ctx, q, out, cache, table, heads: int, kv_heads: int, head_di
             cols = decode_tiles.shape[0] * (16 // hp) * heads
             ws = (take((cols * splits * v_dim,), torch.float32), take((cols * splits * 2,), torch.float32))
         ops.attention_wide(q, out, cache.k, cache.v, decode_tiles, table, heads, kv_heads, head_dim, v_dim, scale, window=window, hp=hp,
-                           splits=splits, workspace=ws, qt=1, slope_exp=slope_exp)
+                           splits=splits, workspace=ws, qt=1, slope_exp=slope_exp, sink_logits=sink_logits)
     return out
 
 
@@ -407,16 +407,16 @@ class Attention:
             ops.unit_kv_write(qkv, ctx.positions, ctx.token_req, table, cache.k, cache.v, s.heads, s.kv_heads, s.head_dim, s.v_dim,
                               s.qk_norm_eps, own_kv=s.own_kv)
         att = ctx.arena.take((n, s.heads * s.v_dim), x.dtype)
-        if s.v_dim == s.head_dim and not s.slope_exp and not s.sink_name and ops.mfma_attention_takes(x.dtype, s.head_dim, cache.k.shape[2]):
+        if s.v_dim == s.head_dim and not s.slope_exp and ops.mfma_attention_takes(x.dtype, s.head_dim, cache.k.shape[2]):
             # bfloat16 on the matrix cores: the tile kernels honour chunks, capped scores and the sink
             for plan in launch_plans(ctx, s.heads // s.kv_heads, s.kv_heads, s.head_dim, span=s.chunk):
                 ops.attention_mfma(qkv, att, cache.k, cache.v, plan.tiles, table, s.heads, s.kv_heads, s.head_dim, s.softmax_scale,
                                    window=s.window, hp=plan.hp, splits=plan.splits, workspace=plan.workspace, qt=plan.qt, coop=plan.coop,
-                                   chunk=s.chunk, cap=s.score_cap, sink=s.sink)
-        elif not (s.chunk or s.score_cap or s.sink or s.sink_name) and ops.wide_attention_takes(x.dtype, s.head_dim, s.v_dim, cache.k.shape[2]):
+                                   chunk=s.chunk, cap=s.score_cap, sink=s.sink, sink_logits=self.sink_logits)
+        elif not (s.chunk or s.score_cap or s.sink) and ops.wide_attention_takes(x.dtype, s.head_dim, s.v_dim, cache.k.shape[2]):
             # bfloat16, values of another size than the keys or a bias by distance: the two-size matrix-core kernel
             wide_attention(ctx, qkv, att, cache, table, s.heads, s.kv_heads, s.head_dim, s.v_dim, s.softmax_scale, window=s.window,
-                           slope_exp=s.slope_exp)
+                           slope_exp=s.slope_exp, sink_logits=self.sink_logits)
         else:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads, s.head_dim,
                                   s.softmax_scale, window=s.window, v_dim=s.v_dim, chunk=s.chunk, cap=s.score_cap, sink=s.sink,

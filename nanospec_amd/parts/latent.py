@@ -124,8 +124,8 @@ class LatentAttention:
             ops.headwise_product(q, D + R, self.uk, q_lat, C + R)
         ops.latent_q_absorb(q, None if self._mfma_q else self.uk, pos.inv_freq, self._factor, ctx.positions, H, D, R, C, out=q_lat)
         o_lat = take((n, H * C), x.dtype)
-        if self.sink_logits is None and ops.wide_attention_takes(x.dtype, C + R, C, cache.k.shape[2]):
-            wide_attention(ctx, q_lat, o_lat, cache, table, H, 1, C + R, C, s.softmax_scale, window=s.window)
+        if ops.wide_attention_takes(x.dtype, C + R, C, cache.k.shape[2]):
+            wide_attention(ctx, q_lat, o_lat, cache, table, H, 1, C + R, C, s.softmax_scale, window=s.window, sink_logits=self.sink_logits)
         else:
             ops.attention_generic(q_lat, o_lat, cache.k, cache.v, ctx.token_req, ctx.positions, table, H, 1, C + R, s.softmax_scale,
                                   window=s.window, v_dim=C, sink_logits=self.sink_logits)

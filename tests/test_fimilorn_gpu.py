@@ -173,7 +173,7 @@ def close(ours, ref, dtype, what, loose=None):
         assert err.max() <= 0.15 and (len(err) < 8 or err.median() <= 0.08), f"{what}: {err.max():.3f} of the logits' spread (median {err.median():.3f})"
 
 
-def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True):
+def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True, loose_share=10):
     from nanospec_amd.engine.replay import Replayer
 
     rep = Replayer(model, max_tokens, page_size=page, use_graphs=graphs)
@@ -200,7 +200,7 @@ def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True):
             close(out, torch.stack([ref[rid][p] for rid, p in w]), dtype, f"step {step['step']} {[(e['id'], len(e['tokens'])) for e in step['entries']]}", loose)
     # (a model here asks its routers four to eight times a token, each time with a chance of a few per cent that bfloat16 rounding
     # moves a close call; such a row then differs by more than rounding)
-    assert len(loose) <= max(2, rows // 10), f"{len(loose)} of {rows} rows are off by more than rounding: {loose[:5]}"
+    assert len(loose) <= max(2, rows // loose_share), f"{len(loose)} of {rows} rows are off by more than rounding: {loose[:5]}"
     rep.manager.check()
     rep.pages_again = sum(1 for who in holders.values() if len(who) > 1)
     rep.slots_again = sum(1 for who in slots.values() if len({r for r in who if r != "__pad__"}) > 1)
@@ -407,7 +407,9 @@ def drawn_config(seed: int) -> dict:
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("seed", range(8))
 def test_drawn_configurations_match_plain(tmp_path, seed, dtype):
-    """Eight configurations drawn at random: in portions, then in a mixed batch, in a small pool."""
+    """Eight configurations drawn at random: in portions, then in a mixed batch, in a small pool.  (Some of them choose one
+    expert of a few, or all experts from one group of two: there a close call that bfloat16 rounding moves changes a row
+    altogether, so more rows may differ by more than rounding.)"""
     from nanospec_amd.loader import load_model
 
     cfg = drawn_config(seed)
@@ -418,9 +420,9 @@ def test_drawn_configurations_match_plain(tmp_path, seed, dtype):
     ref = {rid: pf.forward(cfg, w, toks).float() for rid, toks in seqs.items()}
     page = [4, 8, 16][seed % 3]
     steps, where = traces.portions(seqs, seed=seed)
-    replay(model, steps, where, ref, dtype, 192, page)
+    replay(model, steps, where, ref, dtype, 192, page, loose_share=5)
     steps, where, peak = traces.mixed(seqs, seed=seed, max_live=3)
-    replay(model, steps, where, ref, dtype, peak, page)
+    replay(model, steps, where, ref, dtype, peak, page, loose_share=5)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
@@ -775,3 +777,92 @@ def test_what_a_pass_adds_to_the_stream(W):
         if use_vec:
             want = want + vec.float()
         assert torch.equal(x.cpu(), want)
+
+
+def step_context(lens, starts, tables):
+    """The framework's own batch builder for hand-made requests: tables[b] lists the pages of request b."""
+    import numpy as np
+
+    from nanospec_amd.engine.arena import Arena
+    from nanospec_amd.engine.context import BatchLayout, StepContext, fill_batch
+    from nanospec_amd.parts.attention import TILES
+
+    width = max(len(t) for t in tables)
+    layout = BatchLayout(sum(lens), len(lens), 0, 1, width, plans=[(TILES, TILES.shape(lens))])
+    host = np.zeros(layout.total, dtype=np.int32)
+    table = np.full((len(lens), width), -1, dtype=np.int32)
+    for b, t in enumerate(tables):
+        table[b, : len(t)] = t
+    fill_batch(host, layout, [0] * sum(lens), starts, lens, list(range(len(lens))), [], [table])
+    max_kv = max(s + n for s, n in zip(starts, lens))
+    chunk_kv = max((s + n for s, n in zip(starts, lens) if n != 1), default=0)
+    return StepContext(layout, torch.from_numpy(host).to(DEV), Arena(DEV), max_position=max_kv - 1, max_kv_len=max_kv, max_chunk_kv=chunk_kv)
+
+
+@pytest.mark.parametrize("HD,VD,page,H,G,window", [(48, 32, 8, 4, 2, 37), (80, 64, 16, 3, 1, 0), (96, 64, 16, 4, 1, 136), (64, 64, 16, 8, 2, 0),
+                                                   (32, 32, 8, 2, 2, 20), (128, 128, 16, 4, 1, 0)])
+def test_learned_sinks_on_the_matrix_cores(HD, VD, page, H, G, window):
+    """The matrix-core attention kernels (keys and values of one size, and of two) with a learned sink per head: a prompt
+    portion behind cached keys beside three single tokens of other requests, the keys in one range and cut into ranges that a
+    second kernel joins; against the plain soft-max with the sink's term, and against the plain kernel."""
+    from nanospec_amd.kernels import ops
+    from nanospec_amd.parts.attention import TilePlan
+
+    g = torch.Generator().manual_seed(HD + VD)
+    lens, starts = [45, 1, 1, 1], [150, 0, 299, 64]
+    total = [s + n for s, n in zip(starts, lens)]
+    pages_of = [-(-t // page) for t in total]
+    ids = list(range(sum(pages_of)))
+    random.Random(3).shuffle(ids)
+    tables, at = [], 0
+    for n in pages_of:
+        tables.append(ids[at : at + n])
+        at += n
+    ks = [torch.randn(t, G, HD, generator=g).to(torch.bfloat16) for t in total]
+    vs = [torch.randn(t, G, VD, generator=g).to(torch.bfloat16) for t in total]
+    kc, vc = torch.zeros(len(ids), G, page, HD, dtype=torch.bfloat16), torch.zeros(len(ids), G, VD, page, dtype=torch.bfloat16)
+    for b, tab in enumerate(tables):
+        for t in range(total[b]):
+            kc[tab[t // page], :, t % page] = ks[b][t]
+            vc[tab[t // page], :, :, t % page] = vs[b][t]
+    kc, vc = kc.to(DEV), vc.to(DEV)
+    n = sum(lens)
+    q = torch.randn(n, H, HD, generator=g).to(torch.bfloat16)
+    sink = torch.linspace(-2.0, 5.0, H)  # from a sink that hardly counts to one that takes most of the weight
+    ctx = step_context(lens, starts, tables)
+    scale = 1.5 / math.sqrt(HD)
+    refs, row = [], 0
+    for b, m in enumerate(lens):
+        pos = torch.arange(starts[b], starts[b] + m)
+        dist = pos[:, None] - torch.arange(total[b])[None, :]
+        mask = (dist >= 0) & ((dist < window) if window else (dist >= 0))
+        out = torch.zeros(m, H, VD, dtype=torch.float64)
+        for h in range(H):
+            s = (q[row : row + m, h].double() @ ks[b][:, h // (H // G)].double().T) * scale
+            out[:, h] = pf.sink_softmax(s.masked_fill(~mask, float("-inf")), sink[h]) @ vs[b][:, h // (H // G)].double()
+        refs.append(out)
+        row += m
+    ref = torch.cat(refs).reshape(n, H * VD)
+    assert (ref.abs().view(n, H, VD).amax(-1).amin(0) < 0.7 * ref.abs().view(n, H, VD).amax(-1).amax(0)).any(), "the sinks were meant to take weight"
+    chunk_tiles, decode_tiles = TilePlan.views(ctx)
+    hp = 1
+    while hp < min(H // G, 16):
+        hp *= 2
+    qd = q.reshape(n, H * HD).to(DEV)
+    table = ctx.block_tables[0]
+    for splits in (1, 3):
+        out = torch.zeros(n, H * VD, dtype=torch.bfloat16, device=DEV)
+        for tiles, kw in ((chunk_tiles, dict(hp=1, qt=2)), (decode_tiles, dict(hp=hp, qt=1))):
+            cols = tiles.shape[0] * (kw["qt"] * 16 // kw["hp"]) * H
+            ws = (torch.zeros(cols * splits * VD, device=DEV), torch.zeros(cols * splits * 2, device=DEV)) if splits > 1 else None
+            if HD == VD:
+                ops.attention_mfma(qd, out, kc, vc, tiles, table, H, G, HD, scale, window=window, splits=splits, workspace=ws, sink_logits=sink.to(DEV),
+                                   coop=kw["qt"] == 1, **kw)
+            else:
+                ops.attention_wide(qd, out, kc, vc, tiles, table, H, G, HD, VD, scale, window=window, splits=splits, workspace=ws,
+                                   sink_logits=sink.to(DEV), **kw)
+        err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+        assert err <= 0.02, (splits, err)
+    plain = torch.zeros(n, H * VD, dtype=torch.bfloat16, device=DEV)
+    ops.attention_generic(qd, plain, kc, vc, ctx.token_req, ctx.positions, table, H, G, HD, scale, window=window, v_dim=VD, sink_logits=sink.to(DEV))
+    assert (plain.cpu().double() - ref).abs().max() / ref.abs().max() <= 0.02
