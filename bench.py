@@ -329,7 +329,11 @@ def design_compare(a) -> int:
     out = {}
     k = min(a.steps, 128)
     beside = [(CLOSEST[design], DESIGNS[CLOSEST[design]](shape))] if design in CLOSEST else []
-    for name, cfg in (("llama", llama), *beside, (design, vz)):
+    if a.alone:  # (for profiles of the design's own kernels)
+        llama_first, beside = [], []
+    else:
+        llama_first = [("llama", llama)]
+    for name, cfg in (*llama_first, *beside, (design, vz)):
         model = random_model(cfg, seed=0, dtype=dtype, on_device=True)
         facts = types.SimpleNamespace(vocab_size=shape["vocab_size"])
         row = {}
@@ -343,6 +347,10 @@ def design_compare(a) -> int:
         out[name] = row
         del model
         torch.cuda.empty_cache()
+    if a.alone:
+        print(json.dumps({"metric": f"prefill and decode tok/s of the {design.capitalize()} design at the {SHAPE_NAMES[a.shape]} ({a.dtype})",
+                          "unit": "tok/s", "n_gpus": 1, "dtype": a.dtype, design: out[design]}), flush=True)
+        return 0
     ratio = {key: round(out[design][key] / out["llama"][key], 3) for key in out["llama"] if key.endswith("tok_s")}
     layers = [l.type + ("*" if getattr(l, "kv_from", None) is not None else "") for l in vz.layers]
     print(json.dumps({"metric": f"prefill and decode tok/s of the {design.capitalize()} design beside Llama at the {SHAPE_NAMES[a.shape]} ({a.dtype})",
@@ -374,6 +382,7 @@ def main() -> int:
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="the benchmark's shape is 8b; the others are for profiles")
     ap.add_argument("--design", default=None, choices=sorted(DESIGNS),
                     help="instead of the benchmark: prefill and decode of this design beside the Llama model of the same --shape")
+    ap.add_argument("--alone", action="store_true", help="with --design: that design only, without the models it is measured beside")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (--gpus must be 1)")
