@@ -78,7 +78,9 @@ class LatentAttention:
         # the two per-head matrices, each in the layout its kernel walks: on the matrix cores (bfloat16, sizes that fit) every
         # head's matrix as [out, in] rows; otherwise as the plain kernels of ``csrc/latent.hip`` read them
         D, R, E, C = s.head_dim, s.rot_dim, s.value_dim, s.kv_rank
-        self._mfma_q = ops.headwise_takes(dtype, C, D, D + R, C + R) and s.hidden % 8 == 0 and s.q_rank % 8 == 0 and self.q_cols % 8 == 0
+        # (without a query latent the queries are columns of the first product's rows, which must then start 16 bytes apart)
+        self._mfma_q = (ops.headwise_takes(dtype, C, D, D + R, C + R) and s.hidden % 8 == 0 and s.q_rank % 8 == 0
+                        and (s.q_rank > 0 or self.first.n % 8 == 0))
         self._mfma_o = ops.headwise_takes(dtype, E, C, C, E)
         uk, uv = to(n["uk"]), to(n["uv"])
         self.uk = uk.view(s.heads, D, C).transpose(1, 2).contiguous() if self._mfma_q else uk  # [heads, latent, dim] | [heads * dim, latent]

@@ -866,3 +866,47 @@ def test_learned_sinks_on_the_matrix_cores(HD, VD, page, H, G, window):
     plain = torch.zeros(n, H * VD, dtype=torch.bfloat16, device=DEV)
     ops.attention_generic(qd, plain, kc, vc, ctx.token_req, ctx.positions, table, H, G, HD, scale, window=window, v_dim=VD, sink_logits=sink.to(DEV))
     assert (plain.cpu().double() - ref).abs().max() / ref.abs().max() <= 0.02
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("H,D,R,E,C,window", [(3, 24, 8, 40, 56, 50), (1, 16, 2, 48, 16, 7), (8, 32, 16, 16, 64, 0), (2, 32, 32, 64, 96, 17), (5, 64, 32, 48, 96, 1)])
+def test_latent_attention_without_a_query_latent_over_six_steps(dtype, H, D, R, E, C, window):
+    """The mixer alone over a paged cache whose pages are not in order: a prompt portion, a second one, then single tokens and
+    short portions, so that the window passes over decoded tokens and over the cuts; queries projected from the input itself,
+    learned sinks; against the plain mixer over the whole sequence."""
+    from nanospec_amd.cache.storage import PagedView
+    from nanospec_amd.config.spec import LatentAttentionSpec, RopeSpec
+    from nanospec_amd.parts.latent import LatentAttention
+
+    Wd, T, page = 72, 90, 8
+    spec = LatentAttentionSpec(hidden=Wd, heads=H, head_dim=D, rot_dim=R, value_dim=E, q_rank=0, kv_rank=C, position=RopeSpec(rotary_dim=R, theta=1000.0),
+                               softmax_scale=0.3, norm_eps=1e-5, window=window, gate=False, names=("", "", "q", "dkv", "dkv.norm", "uk", "uv", "", "o"),
+                               sink_name="sink")
+    part = LatentAttention(spec, "m.")
+    g = torch.Generator().manual_seed(H * D + R)
+    w = {}
+    for name, (shape, role) in part.wanted().items():
+        w[name] = (torch.randn(shape, generator=g) * (0.3 if role == "linear" else 1.0)).to(dtype)
+    assert set(w) == {"m." + n for n in ("q", "dkv", "dkv.norm", "uk", "uv", "o", "sink")}
+    part.load(lambda name: w[name], dtype, DEV)
+    x = torch.randn(T, Wd, generator=g).to(dtype)
+    m = dict(heads=H, dim=D, rot_dim=R, vdim=E, kv_rank=C, scale=0.3, rot={"dims": R, "base": 1000.0})
+    if window:
+        m["mask"] = {"size": window}
+    ref = pf.latent_attention(x.double(), {k: v.double() for k, v in w.items()}, "m.", m, 1e-5, torch.arange(T))
+    pages = -(-T // page)
+    order = list(range(pages))
+    random.Random(2).shuffle(order)
+    cache = PagedView(0, torch.zeros(pages, 1, page, C + R, dtype=dtype, device=DEV), torch.zeros(pages, 1, C, page, dtype=dtype, device=DEV))
+    got, at = [], 0
+    for n in (37, 30, 1, 1, 2, 19):
+        ctx = step_context([n], [at], [order])
+        got.append(part.forward(ctx, x[at : at + n].to(DEV), cache, True).cpu())
+        at += n
+    got = torch.cat(got).double()
+    if dtype == torch.float32:
+        err = (got - ref).abs().max() / ref.abs().max()
+        assert err <= 2e-5, err
+    else:  # (sharp soft-maxes magnify a rounding in single places: the root mean square is what bfloat16 is held to)
+        err = (got - ref).pow(2).mean().sqrt() / ref.pow(2).mean().sqrt()
+        assert err <= 0.03, err
