@@ -279,8 +279,8 @@ def padetar_config(shape: dict, layers: int | None = None):
 # of k, learned sinks, an output gate), latent attention (the shape's heads with head_dim unrotated and head_dim / 2 rotated
 # channels, a latent of 512, windows of 1,024, learned sinks), retention (width / 256 heads of 128 key and 256 value channels).
 # The first layer's feed-forward is the clipped dense one of the shape's inner size; every other is 32 experts of an eighth of
-# it in 8 groups of which 4 are kept, four experts a token, beside a shared expert of half the inner size.  The first three
-# layers run twice, and the model has three layers fewer than the shape, so that a token passes as many layers.
+# it in 8 groups of which 4 are kept, four experts a token, beside a shared expert of half the inner size.  The three layers
+# behind the first run twice, and the model has three layers fewer than the shape, so that a token passes as many layers.
 def fimilorn_config(shape: dict, layers: int | None = None):
     from nanospec_amd.config import FimilornConfig
 
@@ -298,7 +298,7 @@ def fimilorn_config(shape: dict, layers: int | None = None):
     entries = [{"type": mixers[i % 3][0], "mixer": mixers[i % 3][1], "mlp": {"kind": "dense", "ff": ff, "limit": 7.0} if i == 0 else moe}
                for i in range(n)]
     return FimilornConfig.from_hf({"architecture": "Fimilorn", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6},
-                                   "loop": {"start": 0, "stop": 3, "times": 2}, "layers": entries})
+                                   "loop": {"start": 1, "stop": 4, "times": 2}, "layers": entries})
 
 
 DESIGNS = {"vuzelix": vuzelix_config, "fetitar": fetitar_config, "padetar": padetar_config, "fimilorn": fimilorn_config}

@@ -52,6 +52,49 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(const T* __restrict__ h
   }
 }
 
+// The same logits for a step of few tokens (up to ROUTE_TOK): a workgroup an expert, its four waves a quarter of the row each
+// (a wave alone walks a row of 2,048 columns in eight dependent rounds; four waves in two), their sums joined in LDS in a
+// fixed order.  A token's logit does not depend on how many tokens the step holds.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_logits_few_kernel(const T* __restrict__ h, int h_stride, const float* __restrict__ wr,
+                                                             const float* __restrict__ br, float* __restrict__ z, int n, int W, int experts, int vec) {
+  __shared__ float part[4][ROUTE_TOK];
+  const int e = blockIdx.x, lane = threadIdx.x % NS_WAVE, wave = threadIdx.x / NS_WAVE;
+  const float* w = wr + (size_t)e * W;
+  float acc[ROUTE_TOK];
+#pragma unroll
+  for (int i = 0; i < ROUTE_TOK; ++i) acc[i] = 0.f;
+  if (vec) {
+    for (int c = threadIdx.x * 4; c < W; c += 256 * 4) {
+      const float4 wc = *reinterpret_cast<const float4*>(w + c);
+#pragma unroll
+      for (int i = 0; i < ROUTE_TOK; ++i)
+        if (i < n) {
+          const T* x = h + (size_t)i * h_stride + c;
+          acc[i] = fmaf(to_f(x[0]), wc.x, acc[i]), acc[i] = fmaf(to_f(x[1]), wc.y, acc[i]);
+          acc[i] = fmaf(to_f(x[2]), wc.z, acc[i]), acc[i] = fmaf(to_f(x[3]), wc.w, acc[i]);
+        }
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += 256) {
+      const float wc = w[c];
+#pragma unroll
+      for (int i = 0; i < ROUTE_TOK; ++i)
+        if (i < n) acc[i] = fmaf(to_f(h[(size_t)i * h_stride + c]), wc, acc[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < ROUTE_TOK; ++i) {
+    const float v = wave_sum(acc[i]);
+    if (lane == 0) part[wave][i] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x < n) {
+    const int i = threadIdx.x;
+    z[(size_t)i * experts + e] = ((part[0][i] + part[1][i]) + (part[2][i] + part[3][i])) + (br ? br[e] : 0.f);
+  }
+}
+
 // A wave a token: the choice scores in LDS, every lane looks through its share for the largest one not yet taken, the lanes'
 // candidates meet by lane exchange (the larger value wins, the lower index among equals; what is no number counts as
 // minus infinity, so a row of anything still chooses ``top`` different experts).
@@ -152,12 +195,16 @@ extern "C" int ns_moe_route(const void* h, int h_stride, const float* wr, const 
   if (grid.y > 65535) return NS_ERR_UNSUPPORTED;
   const size_t elem = dtype == NS_DTYPE_F32 ? 4 : 2;
   const int vec = W % 4 == 0 && h_stride % 4 == 0 && (uintptr_t)wr % 16 == 0 && (uintptr_t)h % (4 * elem) == 0;
-  if (dtype == NS_DTYPE_F32)
+  if (dtype != NS_DTYPE_F32 && dtype != NS_DTYPE_BF16) return NS_ERR_UNSUPPORTED;
+  if (n <= ROUTE_TOK) {  // few tokens: a workgroup an expert
+    if (dtype == NS_DTYPE_F32)
+      moe_logits_few_kernel<float><<<experts, 256, 0, stream>>>((const float*)h, h_stride, wr, br, z, n, W, experts, vec);
+    else
+      moe_logits_few_kernel<bf16_t><<<experts, 256, 0, stream>>>((const bf16_t*)h, h_stride, wr, br, z, n, W, experts, vec);
+  } else if (dtype == NS_DTYPE_F32)
     moe_logits_kernel<float><<<grid, 256, 0, stream>>>((const float*)h, h_stride, wr, br, z, n, W, experts, vec);
-  else if (dtype == NS_DTYPE_BF16)
-    moe_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)h, h_stride, wr, br, z, n, W, experts, vec);
   else
-    return NS_ERR_UNSUPPORTED;
+    moe_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)h, h_stride, wr, br, z, n, W, experts, vec);
   moe_choose_kernel<<<n, 64, 0, stream>>>(z, sel, wt, n, experts, top, sigmoid, correction, groups, keep);
   return ns_launch_status();
 }
