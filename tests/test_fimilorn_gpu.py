@@ -804,7 +804,8 @@ def step_context(lens, starts, tables):
 def test_learned_sinks_on_the_matrix_cores(HD, VD, page, H, G, window):
     """The matrix-core attention kernels (keys and values of one size, and of two) with a learned sink per head: a prompt
     portion behind cached keys beside three single tokens of other requests, the keys in one range and cut into ranges that a
-    second kernel joins; against the plain soft-max with the sink's term, and against the plain kernel."""
+    second kernel joins, with keys that stand out just inside and just outside the window of a prompt's row and of a decoded
+    row; against the plain soft-max with the sink's term, and against the plain kernel."""
     from nanospec_amd.kernels import ops
     from nanospec_amd.parts.attention import TilePlan
 
@@ -820,14 +821,23 @@ def test_learned_sinks_on_the_matrix_cores(HD, VD, page, H, G, window):
         at += n
     ks = [torch.randn(t, G, HD, generator=g).to(torch.bfloat16) for t in total]
     vs = [torch.randn(t, G, VD, generator=g).to(torch.bfloat16) for t in total]
-    kc, vc = torch.zeros(len(ids), G, page, HD, dtype=torch.bfloat16), torch.zeros(len(ids), G, VD, page, dtype=torch.bfloat16)
-    for b, tab in enumerate(tables):
-        for t in range(total[b]):
-            kc[tab[t // page], :, t % page] = ks[b][t]
-            vc[tab[t // page], :, :, t % page] = vs[b][t]
-    kc, vc = kc.to(DEV), vc.to(DEV)
     n = sum(lens)
     q = torch.randn(n, H, HD, generator=g).to(torch.bfloat16)
+    # keys that the last query of the portion and the decoded token of the third request like best: the last one that their
+    # window still holds and the first one it no longer holds (without a window: one far back and one at a page's first place)
+    row = 0
+    for bq, m in enumerate(lens):
+        last = total[bq] - 1
+        for key in ({last - window + 1, last - window} if window else {3, (last // page) * page}):
+            if 0 <= key < last and bq in (0, 2):
+                ks[bq][key] = (4.0 * q[row + m - 1].view(G, H // G, HD)[:, 0].float() / math.sqrt(HD)).to(torch.bfloat16)
+        row += m
+    kc, vc = torch.zeros(len(ids), G, page, HD, dtype=torch.bfloat16), torch.zeros(len(ids), G, VD, page, dtype=torch.bfloat16)
+    for bq, tab in enumerate(tables):
+        for t in range(total[bq]):
+            kc[tab[t // page], :, t % page] = ks[bq][t]
+            vc[tab[t // page], :, :, t % page] = vs[bq][t]
+    kc, vc = kc.to(DEV), vc.to(DEV)
     sink = torch.linspace(-2.0, 5.0, H)  # from a sink that hardly counts to one that takes most of the weight
     ctx = step_context(lens, starts, tables)
     scale = 1.5 / math.sqrt(HD)
