@@ -800,7 +800,8 @@ def step_context(lens, starts, tables):
 
 
 @pytest.mark.parametrize("HD,VD,page,H,G,window", [(48, 32, 8, 4, 2, 37), (80, 64, 16, 3, 1, 0), (96, 64, 16, 4, 1, 130), (64, 64, 16, 8, 2, 0),
-                                                   (32, 32, 8, 2, 2, 20), (128, 128, 16, 4, 1, 0)])
+                                                   (32, 32, 8, 2, 2, 20), (128, 128, 16, 4, 1, 0), (48, 32, 16, 6, 2, 0), (64, 64, 16, 6, 2, 50),
+                                                   (80, 64, 16, 12, 1, 33)])
 def test_learned_sinks_on_the_matrix_cores(HD, VD, page, H, G, window):
     """The matrix-core attention kernels (keys and values of one size, and of two) with a learned sink per head: a prompt
     portion behind cached keys beside three single tokens of other requests, the keys in one range and cut into ranges that a
